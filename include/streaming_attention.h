@@ -1,0 +1,116 @@
+/* C ABI of libstreaming_attention.so -- hand-written gfx950 (MI355X) kernels for
+ * chunk-windowed ("streaming") attention, forward and backward.
+ *
+ * This is the seam at which the reference launches its Triton kernels; every entry
+ * point cites the reference launch it replaces (paths relative to the reference
+ * repository).  The reference has no FFI of its own (it is Python + a run-time
+ * compiled DSL), so the binding on its side is a ctypes stub.
+ *
+ * Common rules
+ *   - Every pointer is a device pointer owned by the caller.  Nothing is allocated,
+ *     freed or synchronised here: each call enqueues kernels on `stream` (a hipStream_t,
+ *     NULL = the default stream) and returns.
+ *   - q/k/v/dO/o inputs are [B,H,T,D] with element strides given as int64[4]
+ *     (batch, head, time, dim).  The dim stride must be 1; base pointers must be
+ *     16-byte aligned and the other strides multiples of 16 bytes.  Outputs are
+ *     written contiguous [B,H,T,D] (lse/delta: contiguous [B,H,T] float32).
+ *   - dtype: 0 = float32, 1 = float16, 2 = bfloat16.  D in {16,32,64,128,256}.
+ *   - lens: int32 per batch entry (may be NULL = every sequence has length T);
+ *     lens_stride in elements; values are clamped to [0, T].
+ *   - Outputs are fully written, including the zeros at positions t >= lens[b];
+ *     the caller need not clear them first.
+ *   - Return value: 0 on success, > 0 a hipError_t from the launch, < 0 one of SA_ERR_*.
+ *   - Re-entrant; no global mutable state apart from one-time kernel attribute set-up.
+ */
+#ifndef STREAMING_ATTENTION_H
+#define STREAMING_ATTENTION_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SA_DTYPE_F32 0
+#define SA_DTYPE_F16 1
+#define SA_DTYPE_BF16 2
+
+#define SA_ERR_DTYPE (-1)
+#define SA_ERR_HEAD_DIM (-2)
+#define SA_ERR_ARG (-3)
+#define SA_ERR_LAYOUT (-4)
+#define SA_ERR_TOO_LARGE (-5)
+
+/* Forward pass: O = softmax_window(sm_scale * Q K^T) V, LSE = log2 sum exp (scaled scores).
+ * Replaces the launch of `_streaming_attn_fwd` inside `attention_forward_adapter`
+ * (src/streaming_attention/kernel.py:1302-1333; kernel at :196-430).
+ * `lse` may be NULL when the caller does not need it. */
+int sa_forward(const void* q, const void* k, const void* v,
+               const int32_t* lens, int64_t lens_stride,
+               void* o, float* lse,
+               const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+               int B, int H, int T, int D,
+               int context_size, int back_contexts, float sm_scale,
+               int dtype, void* stream);
+
+/* delta[b,h,t] = sum_d O * dO in float32.
+ * Replaces the launch of `_streaming_attn_bwd_precompute`
+ * (src/streaming_attention/kernel.py:1380-1397; kernel at :433-514). */
+int sa_bwd_delta(const void* o, const void* d_o, float* delta,
+                 const int64_t* o_strides, const int64_t* do_strides,
+                 int B, int H, int T, int D, int dtype, void* stream);
+
+/* dQ.  Replaces the dQ workers of the fused launch `_streaming_attn_bwd`
+ * (src/streaming_attention/kernel.py:1403-1440; workers at :638-773 and :940-1023). */
+int sa_bwd_dq(const void* q, const void* k, const void* v,
+              const int32_t* lens, int64_t lens_stride,
+              const void* d_o, const float* lse, const float* delta,
+              void* dq,
+              const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+              const int64_t* do_strides,
+              int B, int H, int T, int D,
+              int context_size, int back_contexts, float sm_scale,
+              int dtype, void* stream);
+
+/* dK and dV.  Replaces the dK/dV workers of the same fused launch
+ * (src/streaming_attention/kernel.py:1403-1440; workers at :776-937 and :1026-1129). */
+int sa_bwd_dkdv(const void* q, const void* k, const void* v,
+                const int32_t* lens, int64_t lens_stride,
+                const void* d_o, const float* lse, const float* delta,
+                void* dk, void* dv,
+                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                const int64_t* do_strides,
+                int B, int H, int T, int D,
+                int context_size, int back_contexts, float sm_scale,
+                int dtype, void* stream);
+
+/* Whole backward = sa_bwd_delta + sa_bwd_dkdv + sa_bwd_dq on one stream; `delta` is a
+ * caller-provided [B,H,T] float32 workspace.  Replaces the body of
+ * `attention_backward_adapter` (src/streaming_attention/kernel.py:1363-1442). */
+int sa_backward(const void* q, const void* k, const void* v,
+                const int32_t* lens, int64_t lens_stride,
+                const void* o, const void* d_o, const float* lse, float* delta,
+                void* dq, void* dk, void* dv,
+                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                const int64_t* o_strides, const int64_t* do_strides,
+                int B, int H, int T, int D,
+                int context_size, int back_contexts, float sm_scale,
+                int dtype, void* stream);
+
+/* Static facts about the build, answerable without a GPU.  Replaces the reference's
+ * launch-configuration tables (src/streaming_attention/kernel.py:17-85, 1143-1267) as the
+ * place where tile shapes are looked up.
+ *   what = 0: ABI version          1: waves per workgroup
+ *          2: forward key tile (16-bit types)   3: forward key tile (fp32)
+ *          4: dQ key tile          5: dK/dV query tile
+ *          6: queries (or keys) owned by one workgroup
+ *   anything else: -1 */
+int sa_query(int what);
+
+/* Human-readable text for a return code of the functions above (static storage). */
+const char* sa_error_string(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,179 @@
+// extern "C" surface of libstreaming_attention.so: argument checks, parameter packing
+// and dispatch on the element type.  See include/streaming_attention.h for the contract.
+#include "../../include/streaming_attention.h"
+#include "sa_launch.h"
+
+using namespace sa;
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// strides are element counts; dim stride 1, the others whole 16-byte vectors
+int check_layout(const void* p, const int64_t* s, int dtype) {
+  if (!p || !s) return SA_ERR_ARG;
+  const int64_t vec = dtype == SA_DTYPE_F32 ? 4 : 8;
+  if (s[3] != 1) return SA_ERR_LAYOUT;
+  if (!aligned16(p)) return SA_ERR_LAYOUT;
+  for (int i = 0; i < 3; ++i)
+    if (s[i] % vec != 0) return SA_ERR_LAYOUT;
+  return SA_OK;
+}
+
+int check_common(int B, int H, int T, int D, int dtype) {
+  if (dtype < 0 || dtype > 2) return SA_ERR_DTYPE;
+  if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return SA_ERR_HEAD_DIM;
+  if (B < 0 || H < 0 || T < 0) return SA_ERR_ARG;
+  return SA_OK;
+}
+
+// chunk ids only matter below T, so a larger context behaves like T; likewise R
+void clamp_window(int T, int& C, int& R) {
+  if (C > T) C = T;
+  if (R > T) R = T;
+}
+
+template <typename F> int by_dtype(int dtype, F&& f) {
+  switch (dtype) {
+    case SA_DTYPE_F32: return f(float{});
+    case SA_DTYPE_F16: return f(_Float16{});
+    case SA_DTYPE_BF16: return f(__bf16{});
+  }
+  return SA_ERR_DTYPE;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sa_forward(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
+               void* o, float* lse, const int64_t* qs, const int64_t* ks, const int64_t* vs, int B, int H,
+               int T, int D, int context_size, int back_contexts, float sm_scale, int dtype, void* stream) {
+  if (int rc = check_common(B, H, T, D, dtype)) return rc;
+  if (context_size < 1 || back_contexts < 0) return SA_ERR_ARG;
+  if (B == 0 || H == 0 || T == 0) return SA_OK;
+  if (int rc = check_layout(q, qs, dtype)) return rc;
+  if (int rc = check_layout(k, ks, dtype)) return rc;
+  if (int rc = check_layout(v, vs, dtype)) return rc;
+  if (!o || !aligned16(o)) return o ? SA_ERR_LAYOUT : SA_ERR_ARG;
+  FwdParams p{};
+  p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse; p.lens = lens; p.lens_stride = lens_stride;
+  p.q_sb = qs[0]; p.q_sh = qs[1]; p.q_st = qs[2];
+  p.k_sb = ks[0]; p.k_sh = ks[1]; p.k_st = ks[2];
+  p.v_sb = vs[0]; p.v_sh = vs[1]; p.v_st = vs[2];
+  p.B = B; p.H = H; p.T = T; p.C = context_size; p.R = back_contexts;
+  clamp_window(T, p.C, p.R);
+  p.scale_log2e = sm_scale * kLog2e;
+  return by_dtype(dtype, [&](auto tag) { return launch_fwd<decltype(tag)>(p, D, (hipStream_t)stream); });
+}
+
+int sa_bwd_delta(const void* o, const void* d_o, float* delta, const int64_t* os, const int64_t* gs, int B,
+                 int H, int T, int D, int dtype, void* stream) {
+  if (int rc = check_common(B, H, T, D, dtype)) return rc;
+  if (B == 0 || H == 0 || T == 0) return SA_OK;
+  if (int rc = check_layout(o, os, dtype)) return rc;
+  if (int rc = check_layout(d_o, gs, dtype)) return rc;
+  if (!delta) return SA_ERR_ARG;
+  DeltaParams p{};
+  p.o = o; p.d_o = d_o; p.delta = delta;
+  p.o_sb = os[0]; p.o_sh = os[1]; p.o_st = os[2];
+  p.do_sb = gs[0]; p.do_sh = gs[1]; p.do_st = gs[2];
+  p.B = B; p.H = H; p.T = T;
+  return by_dtype(dtype, [&](auto tag) { return launch_delta<decltype(tag)>(p, D, (hipStream_t)stream); });
+}
+
+static int fill_bwd(BwdParams& p, const void* q, const void* k, const void* v, const int32_t* lens,
+                    int64_t lens_stride, const void* d_o, const float* lse, const float* delta,
+                    const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* gs, int B, int H,
+                    int T, int D, int context_size, int back_contexts, float sm_scale, int dtype) {
+  if (int rc = check_common(B, H, T, D, dtype)) return rc;
+  if (context_size < 1 || back_contexts < 0) return SA_ERR_ARG;
+  if (B == 0 || H == 0 || T == 0) return SA_OK;
+  if (int rc = check_layout(q, qs, dtype)) return rc;
+  if (int rc = check_layout(k, ks, dtype)) return rc;
+  if (int rc = check_layout(v, vs, dtype)) return rc;
+  if (int rc = check_layout(d_o, gs, dtype)) return rc;
+  if (!lse || !delta) return SA_ERR_ARG;
+  p.q = q; p.k = k; p.v = v; p.d_o = d_o; p.lse = lse; p.delta = delta;
+  p.lens = lens; p.lens_stride = lens_stride;
+  p.q_sb = qs[0]; p.q_sh = qs[1]; p.q_st = qs[2];
+  p.k_sb = ks[0]; p.k_sh = ks[1]; p.k_st = ks[2];
+  p.v_sb = vs[0]; p.v_sh = vs[1]; p.v_st = vs[2];
+  p.do_sb = gs[0]; p.do_sh = gs[1]; p.do_st = gs[2];
+  p.B = B; p.H = H; p.T = T; p.C = context_size; p.R = back_contexts;
+  clamp_window(T, p.C, p.R);
+  p.scale = sm_scale;
+  p.scale_log2e = sm_scale * kLog2e;
+  return SA_OK;
+}
+
+int sa_bwd_dq(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
+              const void* d_o, const float* lse, const float* delta, void* dq, const int64_t* qs,
+              const int64_t* ks, const int64_t* vs, const int64_t* gs, int B, int H, int T, int D,
+              int context_size, int back_contexts, float sm_scale, int dtype, void* stream) {
+  BwdParams p{};
+  if (int rc = fill_bwd(p, q, k, v, lens, lens_stride, d_o, lse, delta, qs, ks, vs, gs, B, H, T, D,
+                        context_size, back_contexts, sm_scale, dtype))
+    return rc;
+  if (B == 0 || H == 0 || T == 0) return SA_OK;
+  if (!dq || !aligned16(dq)) return dq ? SA_ERR_LAYOUT : SA_ERR_ARG;
+  p.dq = dq;
+  return by_dtype(dtype, [&](auto tag) { return launch_dq<decltype(tag)>(p, D, (hipStream_t)stream); });
+}
+
+int sa_bwd_dkdv(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
+                const void* d_o, const float* lse, const float* delta, void* dk, void* dv,
+                const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* gs, int B, int H,
+                int T, int D, int context_size, int back_contexts, float sm_scale, int dtype, void* stream) {
+  BwdParams p{};
+  if (int rc = fill_bwd(p, q, k, v, lens, lens_stride, d_o, lse, delta, qs, ks, vs, gs, B, H, T, D,
+                        context_size, back_contexts, sm_scale, dtype))
+    return rc;
+  if (B == 0 || H == 0 || T == 0) return SA_OK;
+  if (!dk || !dv) return SA_ERR_ARG;
+  if (!aligned16(dk) || !aligned16(dv)) return SA_ERR_LAYOUT;
+  p.dk = dk; p.dv = dv;
+  return by_dtype(dtype, [&](auto tag) { return launch_dkdv<decltype(tag)>(p, D, (hipStream_t)stream); });
+}
+
+int sa_backward(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
+                const void* o, const void* d_o, const float* lse, float* delta, void* dq, void* dk, void* dv,
+                const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os, const int64_t* gs,
+                int B, int H, int T, int D, int context_size, int back_contexts, float sm_scale, int dtype,
+                void* stream) {
+  if (int rc = sa_bwd_delta(o, d_o, delta, os, gs, B, H, T, D, dtype, stream)) return rc;
+  if (int rc = sa_bwd_dkdv(q, k, v, lens, lens_stride, d_o, lse, delta, dk, dv, qs, ks, vs, gs, B, H, T, D,
+                           context_size, back_contexts, sm_scale, dtype, stream))
+    return rc;
+  return sa_bwd_dq(q, k, v, lens, lens_stride, d_o, lse, delta, dq, qs, ks, vs, gs, B, H, T, D, context_size,
+                   back_contexts, sm_scale, dtype, stream);
+}
+
+int sa_query(int what) {
+  switch (what) {
+    case 0: return 1;
+    case 1: return Cfg<__bf16>::NW;
+    case 2: return Cfg<__bf16>::FWD_TK;
+    case 3: return Cfg<float>::FWD_TK;
+    case 4: return Cfg<__bf16>::DQ_TK;
+    case 5: return Cfg<__bf16>::DKDV_TQ;
+    case 6: return Cfg<__bf16>::NW * 32;
+  }
+  return -1;
+}
+
+const char* sa_error_string(int code) {
+  switch (code) {
+    case SA_OK: return "success";
+    case SA_ERR_DTYPE: return "unsupported dtype id (0 = float32, 1 = float16, 2 = bfloat16)";
+    case SA_ERR_HEAD_DIM: return "head dimension must be one of 16, 32, 64, 128, 256";
+    case SA_ERR_ARG: return "invalid argument (null pointer, negative size, context_size < 1 or back_contexts < 0)";
+    case SA_ERR_LAYOUT: return "unsupported layout (dim stride must be 1; pointers and strides 16-byte aligned)";
+    case SA_ERR_TOO_LARGE: return "problem too large for one launch";
+  }
+  return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+}
+
+}  // extern "C"

@@ -1,0 +1,366 @@
+// Backward kernels.
+//
+//   delta_kernel  delta[b,h,t] = sum_d O*dO      replaces `_streaming_attn_bwd_precompute`
+//                                                (src/streaming_attention/kernel.py:433-514)
+//   dq_kernel     dQ = scale * dS K              replaces `_streaming_attn_bwd_dq(_inner)`
+//                                                (kernel.py:638-773, 940-1023)
+//   dkdv_kernel   dV = P^T dO, dK = scale dS^T Q replaces `_streaming_attn_bwd_dkdv(_inner)`
+//                                                (kernel.py:776-937, 1026-1129)
+// with P = exp2(scale*log2e * Q K^T - LSE), dP = dO V^T, dS = P o (dP - delta).
+//
+// dq_kernel mirrors the forward: a lane owns a query column, so LSE, delta and the key
+// window are per-lane scalars.  dkdv_kernel is its transpose: a workgroup owns 32*NW keys,
+// a lane owns one key column with its query window [qlo, qhi), and the loop runs over the
+// query tiles that can see those keys (kernel.py:1046-1054).  Both kernels write every
+// element of their outputs, zeros included, so the caller does not pre-clear them.
+#pragma once
+#include "sa_common.h"
+
+namespace sa {
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void delta_kernel(const DeltaParams p) {
+  using E = Elem<T>;
+  using Frag = typename E::Frag;
+  constexpr int LPR = D / E::VEC;      // lanes per row, a power of two <= 64
+  constexpr int RPB = 256 / LPR;       // rows per block
+  const int tid = threadIdx.x;
+  const int sub = tid % LPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + tid / LPR;   // flattened (b,h,t)
+  const int64_t total = (int64_t)p.B * p.H * p.T;
+  float acc = 0.0f;
+  if (row < total) {
+    const int t = (int)(row % p.T);
+    const int64_t bh = row / p.T;
+    const int hd = (int)(bh % p.H);
+    const int64_t b = bh / p.H;
+    const T* op = reinterpret_cast<const T*>(p.o) + b * p.o_sb + hd * p.o_sh + (int64_t)t * p.o_st;
+    const T* gp = reinterpret_cast<const T*>(p.d_o) + b * p.do_sb + hd * p.do_sh + (int64_t)t * p.do_st;
+    const Frag a = *reinterpret_cast<const Frag*>(op + sub * E::VEC);
+    const Frag g = *reinterpret_cast<const Frag*>(gp + sub * E::VEC);
+#pragma unroll
+    for (int e = 0; e < E::VEC; ++e) acc += (float)a[e] * (float)g[e];
+  }
+#pragma unroll
+  for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (row < total && sub == 0) p.delta[row] = acc;
+}
+
+template <typename T, int D, int NW, int TK>
+__global__ __launch_bounds__(NW * 64) void dq_kernel(const BwdParams p) {
+  using E = Elem<T>;
+  using G = TileGeom<T, D>;
+  using Frag = typename E::Frag;
+  constexpr int TQ = NW * 32, NT = NW * 64, KBN = TK / 32;
+  constexpr int PITCH = G::PITCH, NF = G::NF, DB = G::DB;
+  constexpr int TILE = TK * PITCH;
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  T* smem = reinterpret_cast<T*>(smem_raw);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int bid = xcd_remap(blockIdx.x, gridDim.x);
+  const int qt = bid % p.n_tiles;
+  const int bh = bid / p.n_tiles;
+  const int hd = bh % p.H, b = bh / p.H;
+  const int T_ = p.T, C = p.C, R = p.R;
+
+  int L = T_;
+  if (p.lens) {
+    L = p.lens[(int64_t)b * p.lens_stride];
+    L = L < 0 ? 0 : (L > T_ ? T_ : L);
+  }
+  const int q0 = qt * TQ;
+  T* dq_base = reinterpret_cast<T*>(p.dq) + (int64_t)bh * T_ * D;
+  const int q_end = q0 + TQ < T_ ? q0 + TQ : T_;
+  if (q0 >= L) {
+    zero_rows<T, D, NT>(dq_base, q0, q_end, tid);
+    return;
+  }
+
+  const int qrow = q0 + wave * 32 + c;
+  const int qe = qrow < L ? qrow : L - 1;
+  const int qchunk = qe / C;
+  const int lo = (qchunk > R ? qchunk - R : 0) * C;
+  const int hi = (qchunk + 1) * C < L ? (qchunk + 1) * C : L;
+  const int wq_first = q0 + wave * 32 < L ? q0 + wave * 32 : L - 1;
+  const int wq_last = q0 + wave * 32 + 31 < L ? q0 + wave * 32 + 31 : L - 1;
+  const int hi_min = (wq_first / C + 1) * C < L ? (wq_first / C + 1) * C : L;
+  const int lo_max = (wq_last / C > R ? wq_last / C - R : 0) * C;
+  const int gq_last = q0 + TQ - 1 < L ? q0 + TQ - 1 : L - 1;
+  const int lo_wg = (q0 / C > R ? q0 / C - R : 0) * C;
+  const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
+  const int kt0 = lo_wg / TK, kt1 = (hi_wg + TK - 1) / TK;
+
+  const float sl2e = fabsf(p.scale_log2e);
+  const bool neg = p.scale_log2e < 0.0f;
+
+  Frag qf[NF], gf[NF];
+  float lse_q, delta_q;
+  {
+    const int qr = qrow < T_ ? qrow : T_ - 1;
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh +
+                  (int64_t)qr * p.q_st;
+    const T* gp = reinterpret_cast<const T*>(p.d_o) + (int64_t)b * p.do_sb + (int64_t)hd * p.do_sh +
+                  (int64_t)qr * p.do_st;
+#pragma unroll
+    for (int g = 0; g < NF; ++g) {
+      qf[g] = *reinterpret_cast<const Frag*>(qp + (g * 2 + h) * E::VEC);
+      if (neg) qf[g] = negate<T>(qf[g]);
+      gf[g] = *reinterpret_cast<const Frag*>(gp + (g * 2 + h) * E::VEC);
+    }
+    // rows past L get P = exp2(-inf) = 0
+    lse_q = qrow < L ? p.lse[(int64_t)bh * T_ + qr] : INFINITY;
+    delta_q = p.delta[(int64_t)bh * T_ + qr];
+  }
+
+  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh;
+  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh;
+
+  f32x16 acc[DB];
+#pragma unroll
+  for (int m = 0; m < DB; ++m)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
+
+  Stager<T, D, TK, NT> sk, sv;
+  sk.load(kbase, p.k_st, kt0 * TK, T_ - 1, tid);
+  sv.load(vbase, p.v_st, kt0 * TK, T_ - 1, tid);
+  sk.store(smem, tid);
+  sv.store(smem + TILE, tid);
+  __syncthreads();
+
+  for (int t = kt0; t < kt1; ++t) {
+    const int cur = (t - kt0) & 1;
+    const T* Kt = smem + cur * 2 * TILE;
+    const T* Vt = Kt + TILE;
+    const bool more = t + 1 < kt1;
+    if (more) {
+      sk.load(kbase, p.k_st, (t + 1) * TK, T_ - 1, tid);
+      sv.load(vbase, p.v_st, (t + 1) * TK, T_ - 1, tid);
+    }
+    const int k0 = t * TK;
+    const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
+
+#pragma unroll
+    for (int kb = 0; kb < KBN; ++kb) {
+      f32x16 s, dp;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[i] = 0.0f, dp[i] = 0.0f;
+#pragma unroll
+      for (int g = 0; g < NF; ++g) mma(s, lds_row_frag<T, PITCH>(Kt, kb * 32 + c, g, h), qf[g]);
+#pragma unroll
+      for (int g = 0; g < NF; ++g) mma(dp, lds_row_frag<T, PITCH>(Vt, kb * 32 + c, g, h), gf[g]);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float pr = fast_exp2(s[i] * sl2e - lse_q);
+        float ds = pr * (dp[i] - delta_q);
+        if (!interior) {
+          const int key = k0 + kb * 32 + crow(i, h);
+          if (key < lo || key >= hi) ds = 0.0f;
+        }
+        s[i] = ds;
+      }
+      // dQ^T[d][q] += K^T dS^T
+      mma_tr<T, PITCH, DB>(acc, Kt, kb, s, lane);
+    }
+
+    if (more) {
+      T* nxt = smem + (cur ^ 1) * 2 * TILE;
+      sk.store(nxt, tid);
+      sv.store(nxt + TILE, tid);
+    }
+    __syncthreads();
+  }
+
+  if (qrow < T_) {
+    if (qrow >= L) {
+#pragma unroll
+      for (int m = 0; m < DB; ++m)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
+    }
+    store_acc_T<T, D, DB>(dq_base + (int64_t)qrow * D, acc, p.scale, h);
+  }
+}
+
+template <typename T, int D, int NW, int TQ>
+__global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
+  using E = Elem<T>;
+  using G = TileGeom<T, D>;
+  using Frag = typename E::Frag;
+  constexpr int TKB = NW * 32, NT = NW * 64, QBN = TQ / 32;
+  constexpr int PITCH = G::PITCH, NF = G::NF, DB = G::DB;
+  constexpr int TILE = TQ * PITCH;
+  // stage layout: [Q tile][dO tile][lse TQ floats][delta TQ floats]
+  constexpr int STAGE_BYTES = 2 * TILE * (int)sizeof(T) + 2 * TQ * (int)sizeof(float);
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int bid = xcd_remap(blockIdx.x, gridDim.x);
+  const int kt = bid % p.n_tiles;
+  const int bh = bid / p.n_tiles;
+  const int hd = bh % p.H, b = bh / p.H;
+  const int T_ = p.T, C = p.C, R = p.R;
+
+  int L = T_;
+  if (p.lens) {
+    L = p.lens[(int64_t)b * p.lens_stride];
+    L = L < 0 ? 0 : (L > T_ ? T_ : L);
+  }
+  const int k0 = kt * TKB;
+  T* dk_base = reinterpret_cast<T*>(p.dk) + (int64_t)bh * T_ * D;
+  T* dv_base = reinterpret_cast<T*>(p.dv) + (int64_t)bh * T_ * D;
+  const int k_end = k0 + TKB < T_ ? k0 + TKB : T_;
+  if (k0 >= L) {
+    zero_rows<T, D, NT>(dk_base, k0, k_end, tid);
+    zero_rows<T, D, NT>(dv_base, k0, k_end, tid);
+    return;
+  }
+
+  // query window [qlo, qhi) of a key: its own chunk and the R chunks after it, below L
+  auto win_lo = [&](int key) { return (key / C) * C; };
+  auto win_hi = [&](int key) {
+    const int64_t e = ((int64_t)(key / C) + R + 1) * (int64_t)C;
+    return e < (int64_t)L ? (int)e : L;
+  };
+  const int krow = k0 + wave * 32 + c;
+  const int ke = krow < L ? krow : L - 1;  // keys past L mimic the last valid key
+  const int qlo = win_lo(ke), qhi = win_hi(ke);
+  const int wk_first = k0 + wave * 32 < L ? k0 + wave * 32 : L - 1;
+  const int wk_last = k0 + wave * 32 + 31 < L ? k0 + wave * 32 + 31 : L - 1;
+  const int qhi_min = win_hi(wk_first), qlo_max = win_lo(wk_last);
+  const int gk_last = k0 + TKB - 1 < L ? k0 + TKB - 1 : L - 1;
+  const int qt0 = win_lo(k0) / TQ, qt1 = (win_hi(gk_last) + TQ - 1) / TQ;
+
+  const float sl2e = fabsf(p.scale_log2e);
+  const bool neg = p.scale_log2e < 0.0f;
+
+  Frag kf[NF], vf[NF];
+  {
+    const int kr = krow < T_ ? krow : T_ - 1;
+    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh +
+                  (int64_t)kr * p.k_st;
+    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh +
+                  (int64_t)kr * p.v_st;
+#pragma unroll
+    for (int g = 0; g < NF; ++g) {
+      kf[g] = *reinterpret_cast<const Frag*>(kp + (g * 2 + h) * E::VEC);
+      if (neg) kf[g] = negate<T>(kf[g]);
+      vf[g] = *reinterpret_cast<const Frag*>(vp + (g * 2 + h) * E::VEC);
+    }
+  }
+
+  const T* qbase = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh;
+  const T* gbase = reinterpret_cast<const T*>(p.d_o) + (int64_t)b * p.do_sb + (int64_t)hd * p.do_sh;
+  const float* lse_base = p.lse + (int64_t)bh * T_;
+  const float* delta_base = p.delta + (int64_t)bh * T_;
+
+  f32x16 dk[DB], dv[DB];
+#pragma unroll
+  for (int m = 0; m < DB; ++m)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
+
+  Stager<T, D, TQ, NT> sq, sg;
+  float r_lse = 0.0f, r_delta = 0.0f;   // thread tid < TQ stages row tid of the tile
+  auto load_rows = [&](int row0) {
+    if (tid < TQ) {
+      int r = row0 + tid;
+      r = r < T_ ? r : T_ - 1;
+      r_lse = lse_base[r];
+      r_delta = delta_base[r];
+    }
+  };
+  auto stage_ptr = [&](int s) { return smem_raw + s * STAGE_BYTES; };
+  auto store_stage = [&](int s) {
+    T* qd = reinterpret_cast<T*>(stage_ptr(s));
+    sq.store(qd, tid);
+    sg.store(qd + TILE, tid);
+    if (tid < TQ) {
+      float* f = reinterpret_cast<float*>(stage_ptr(s) + 2 * TILE * sizeof(T));
+      f[tid] = r_lse;
+      f[TQ + tid] = r_delta;
+    }
+  };
+  static_assert(TQ <= NW * 64, "one thread per staged row");
+
+  sq.load(qbase, p.q_st, qt0 * TQ, T_ - 1, tid);
+  sg.load(gbase, p.do_st, qt0 * TQ, T_ - 1, tid);
+  load_rows(qt0 * TQ);
+  store_stage(0);
+  __syncthreads();
+
+  for (int t = qt0; t < qt1; ++t) {
+    const int cur = (t - qt0) & 1;
+    const T* Qt = reinterpret_cast<const T*>(stage_ptr(cur));
+    const T* Gt = Qt + TILE;
+    const float* lse_t = reinterpret_cast<const float*>(stage_ptr(cur) + 2 * TILE * sizeof(T));
+    const float* delta_t = lse_t + TQ;
+    const bool more = t + 1 < qt1;
+    if (more) {
+      sq.load(qbase, p.q_st, (t + 1) * TQ, T_ - 1, tid);
+      sg.load(gbase, p.do_st, (t + 1) * TQ, T_ - 1, tid);
+      load_rows((t + 1) * TQ);
+    }
+    const int qs = t * TQ;
+    const bool interior = (qs >= qlo_max) && (qs + TQ <= qhi_min);
+
+#pragma unroll
+    for (int qb = 0; qb < QBN; ++qb) {
+      f32x16 s, dp;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[i] = 0.0f, dp[i] = 0.0f;
+      // S[q][key] = Q K^T, dP[q][key] = dO V^T
+#pragma unroll
+      for (int g = 0; g < NF; ++g) mma(s, lds_row_frag<T, PITCH>(Qt, qb * 32 + c, g, h), kf[g]);
+#pragma unroll
+      for (int g = 0; g < NF; ++g) mma(dp, lds_row_frag<T, PITCH>(Gt, qb * 32 + c, g, h), vf[g]);
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_t + qb * 32 + 8 * g4 + 4 * h);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_t + qb * 32 + 8 * g4 + 4 * h);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = 4 * g4 + e;
+          float pr = fast_exp2(s[i] * sl2e - l4[e]);
+          float ds = pr * (dp[i] - d4[e]);
+          if (!interior) {
+            const int qr = qs + qb * 32 + crow(i, h);
+            const bool ok = qr >= qlo && qr < qhi;
+            pr = ok ? pr : 0.0f;
+            ds = ok ? ds : 0.0f;
+          }
+          s[i] = pr;
+          dp[i] = ds;
+        }
+      }
+      // dV^T[d][key] += dO^T P,  dK^T[d][key] += Q^T dS
+      mma_tr<T, PITCH, DB>(dv, Gt, qb, s, lane);
+      mma_tr<T, PITCH, DB>(dk, Qt, qb, dp, lane);
+    }
+
+    if (more) store_stage(cur ^ 1);
+    __syncthreads();
+  }
+
+  if (krow < T_) {
+    if (krow >= L) {
+#pragma unroll
+      for (int m = 0; m < DB; ++m)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
+    }
+    store_acc_T<T, D, DB>(dk_base + (int64_t)krow * D, dk, p.scale, h);
+    store_acc_T<T, D, DB>(dv_base + (int64_t)krow * D, dv, 1.0f, h);
+  }
+}
+
+}  // namespace sa

@@ -1,0 +1,265 @@
+// Shared device-side building blocks for the streaming-attention kernels (gfx950 / CDNA4).
+//
+// Conventions used by every kernel in this directory
+// --------------------------------------------------
+// A wavefront has 64 lanes; lane l is split as c = l & 31 ("owner" index) and h = l >> 5.
+// All matrix products are 32x32 MFMA tiles, D = A*B + C:
+//   * A fragment: lane supplies A[row c][contraction slots of half h]
+//   * B fragment: lane supplies B[contraction slots of half h][col c]
+//   * C fragment: 16 floats per lane, acc[i] is C[row 8*(i/4) + 4*h + (i%4)][col c]
+// Only the pairing of A and B slots matters for correctness, so every fragment that
+// is loaded straight from memory uses the same rule: fragment g of a row covers the
+// contraction indices [g*2*VEC + h*VEC, g*2*VEC + h*VEC + VEC), one 16-byte vector.
+// For 16-bit types VEC = 8 and a fragment feeds one v_mfma_f32_32x32x16_{bf16,f16};
+// for fp32 VEC = 4 and a fragment feeds four v_mfma_f32_32x32x2_f32.
+//
+// The second product of each attention step contracts over the ROW index of a C
+// fragment that was just computed (keys for P*V, queries for P^T*dO ...).  The lane
+// that owns column c of that C fragment already holds exactly the values a B operand
+// needs, so the probabilities never leave registers; the matching A operand is the
+// transpose of a row-major LDS tile, fetched with ds_read_b64_tr_b16 (16-bit) or with
+// scalar LDS reads (fp32).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sa {
+
+#define SA_DEV __device__ __forceinline__
+#define SA_LDS __attribute__((address_space(3)))
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+  static constexpr int VEC = 8;
+  static constexpr bool HALF = true;
+  using Frag = bf16x8;
+  using Quad = bf16x4;
+  static constexpr uint32_t SIGN = 0x80008000u;
+};
+template <> struct Elem<_Float16> {
+  static constexpr int VEC = 8;
+  static constexpr bool HALF = true;
+  using Frag = f16x8;
+  using Quad = f16x4;
+  static constexpr uint32_t SIGN = 0x80008000u;
+};
+template <> struct Elem<float> {
+  static constexpr int VEC = 4;
+  static constexpr bool HALF = false;
+  using Frag = f32x4;
+  using Quad = f32x4;
+  static constexpr uint32_t SIGN = 0x80000000u;
+};
+
+// LDS row pitch in elements: the head dimension (at least one 32-wide block, so that
+// transposed reads of a D=16 tile stay inside the row) plus one 16-byte pad.
+template <typename T, int D> struct TileGeom {
+  static constexpr int DP = D < 32 ? 32 : D;
+  static constexpr int PITCH = DP + Elem<T>::VEC;
+  static constexpr int NF = D / (2 * Elem<T>::VEC);   // row fragments per lane
+  static constexpr int DB = DP / 32;                  // 32-wide blocks along D
+};
+
+SA_DEV void mma(f32x16& acc, bf16x8 a, bf16x8 b) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+}
+SA_DEV void mma(f32x16& acc, f16x8 a, f16x8 b) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+}
+SA_DEV void mma(f32x16& acc, f32x4 a, f32x4 b) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], acc, 0, 0, 0);
+}
+
+// Value held by lane l^32 combined with the lane's own: v_permlane32_swap hands each
+// lane both its own value and its partner's (in an order that depends on the half),
+// which is all a max or a sum needs.
+SA_DEV float half_max(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+SA_DEV float half_sum(float x) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+SA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+template <typename T> SA_DEV typename Elem<T>::Frag negate(typename Elem<T>::Frag f) {
+  u32x4 u = __builtin_bit_cast(u32x4, f);
+  u ^= Elem<T>::SIGN;
+  return __builtin_bit_cast(typename Elem<T>::Frag, u);
+}
+
+// Row of a C fragment that register i of half h holds.
+SA_DEV constexpr int crow(int i, int h) { return 8 * (i >> 2) + 4 * h + (i & 3); }
+
+// Fragment g of row `row` of a row-major LDS tile (contraction along the row).
+template <typename T, int PITCH>
+SA_DEV typename Elem<T>::Frag lds_row_frag(const T* tile, int row, int g, int h) {
+  using Frag = typename Elem<T>::Frag;
+  return *reinterpret_cast<const Frag*>(tile + row * PITCH + (g * 2 + h) * Elem<T>::VEC);
+}
+
+// acc[m] += X^T * P for one 32-row block `rb` of a row-major LDS tile X[rows][cols]:
+//   acc[m][row x][col c] += sum_r X[rb*32 + r][m*32 + x] * P[r][c]
+// where P is a C fragment (its rows are the contraction index).  P is rounded to T
+// before the product, as the operand of a 16-bit MFMA must be.
+template <typename T, int PITCH, int NM>
+SA_DEV void mma_tr(f32x16 (&acc)[NM], const T* X, int rb, const f32x16& P, int lane) {
+  using E = Elem<T>;
+  if constexpr (E::HALF) {
+    const int g16 = lane >> 4, j = lane & 15;
+    const int h = g16 >> 1, mb = (g16 & 1) * 16;
+    // this lane's source address for the transposing read: row (j/4) of a 4-row run,
+    // 4 columns starting at 4*(j%4); the instruction hands lane j column j of the
+    // 4x16 block, i.e. 4 consecutive rows of one column.
+    const T* base = X + (rb * 32 + 4 * h + (j >> 2)) * PITCH + mb + 4 * (j & 3);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      typename E::Frag b;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) b[e] = (T)P[half * 8 + e];
+#pragma unroll
+      for (int m = 0; m < NM; ++m) {
+        const T* p0 = base + (half * 16) * PITCH + m * 32;
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p0));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p0 + 8 * PITCH));
+        s16x8 a8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        mma(acc[m], __builtin_bit_cast(typename E::Frag, a8), b);
+      }
+    }
+  } else {
+    const int c = lane & 31, h = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const T* row = X + (rb * 32 + crow(i, h)) * PITCH + c;
+#pragma unroll
+      for (int m = 0; m < NM; ++m)
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(row[m * 32], P[i], acc[m], 0, 0, 0);
+    }
+  }
+}
+
+// Cooperative copy of a [ROWS][D] row-major global tile into registers and on into an
+// LDS tile.  Rows are clamped to `last_row` so that a ragged final tile reads valid
+// memory (the values are masked by the caller).
+template <typename T, int D, int ROWS, int NT> struct Stager {
+  using E = Elem<T>;
+  using Frag = typename E::Frag;
+  static constexpr int CPR = D / E::VEC;                 // 16-byte chunks per row
+  static constexpr int TOTAL = ROWS * CPR;
+  static constexpr int N = (TOTAL + NT - 1) / NT;
+  static constexpr int PITCH = TileGeom<T, D>::PITCH;
+  Frag regs[N];
+
+  SA_DEV void load(const T* base, int64_t row_stride, int row0, int last_row, int tid) {
+#pragma unroll
+    for (int it = 0; it < N; ++it) {
+      const int ch = tid + it * NT;
+      if (TOTAL % NT == 0 || ch < TOTAL) {
+        const int r = ch / CPR, col = (ch % CPR) * E::VEC;
+        int gr = row0 + r;
+        gr = gr < last_row ? gr : last_row;
+        regs[it] = *reinterpret_cast<const Frag*>(base + (int64_t)gr * row_stride + col);
+      }
+    }
+  }
+  SA_DEV void store(T* tile, int tid) const {
+#pragma unroll
+    for (int it = 0; it < N; ++it) {
+      const int ch = tid + it * NT;
+      if (TOTAL % NT == 0 || ch < TOTAL) {
+        const int r = ch / CPR, col = (ch % CPR) * E::VEC;
+        *reinterpret_cast<Frag*>(tile + r * PITCH + col) = regs[it];
+      }
+    }
+  }
+};
+
+// Hardware hands workgroup i to XCD i % 8.  Renumber so that each XCD receives a
+// contiguous range of logical ids: neighbouring tiles of one (batch, head) then share
+// that XCD's L2 for the keys and values they have in common.
+SA_DEV int xcd_remap(int bid, int n) {
+  const int per = n >> 3, rem = n & 7;
+  const int x = bid & 7, idx = bid >> 3;
+  return x * per + (x < rem ? x : rem) + idx;
+}
+
+// Write four consecutive fp32 values as four elements of T.
+template <typename T> SA_DEV void store4(T* dst, float a, float b, float c, float d) {
+  typename Elem<T>::Quad q;
+  q[0] = (T)a; q[1] = (T)b; q[2] = (T)c; q[3] = (T)d;
+  *reinterpret_cast<typename Elem<T>::Quad*>(dst) = q;
+}
+
+// Zero rows [row0, row1) of a contiguous [*, D] matrix with the whole workgroup.
+template <typename T, int D, int NT> SA_DEV void zero_rows(T* base, int row0, int row1, int tid) {
+  using E = Elem<T>;
+  constexpr int CPR = D / E::VEC;
+  const int total = (row1 - row0) * CPR;
+  typename E::Frag z;
+#pragma unroll
+  for (int e = 0; e < E::VEC; ++e) z[e] = (T)0.0f;
+  for (int ch = tid; ch < total; ch += NT)
+    *reinterpret_cast<typename E::Frag*>(base + (int64_t)row0 * D + (int64_t)ch * E::VEC) = z;
+}
+
+// Transposed store of DB accumulator blocks holding X^T[d][row] into X[row][d]:
+// register group (4 consecutive d) -> one 8- or 16-byte store.
+template <typename T, int D, int DB>
+SA_DEV void store_acc_T(T* row_ptr, const f32x16 (&acc)[DB], float mul, int h) {
+#pragma unroll
+  for (int m = 0; m < DB; ++m)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int d = m * 32 + 8 * g + 4 * h;
+      if (d < D)
+        store4<T>(row_ptr + d, acc[m][4 * g] * mul, acc[m][4 * g + 1] * mul, acc[m][4 * g + 2] * mul,
+                  acc[m][4 * g + 3] * mul);
+    }
+}
+
+struct FwdParams {
+  const void *q, *k, *v;
+  void* o;          // contiguous [B,H,T,D]
+  float* lse;       // contiguous [B,H,T] or null
+  const int32_t* lens;  // null: every sequence has length T
+  int64_t lens_stride;
+  int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, v_sb, v_sh, v_st;  // element strides
+  int B, H, T, C, R;
+  float scale_log2e;  // sm_scale * log2(e); sign carried separately
+  int n_tiles;        // query tiles per (b,h)
+};
+
+struct BwdParams {
+  const void *q, *k, *v, *d_o;
+  const float *lse, *delta;   // contiguous [B,H,T]
+  void *dq, *dk, *dv;         // contiguous [B,H,T,D]
+  const int32_t* lens;
+  int64_t lens_stride;
+  int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, v_sb, v_sh, v_st, do_sb, do_sh, do_st;
+  int B, H, T, C, R;
+  float scale, scale_log2e;
+  int n_tiles;
+};
+
+struct DeltaParams {
+  const void *o, *d_o;
+  float* delta;
+  int64_t o_sb, o_sh, o_st, do_sb, do_sh, do_st;
+  int B, H, T;
+};
+
+}  // namespace sa

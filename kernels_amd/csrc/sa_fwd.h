@@ -1,0 +1,195 @@
+// Forward kernel: O = softmax_window(scale * Q K^T) V and the base-2 log-sum-exp.
+//
+// Replaces the reference's Triton kernel `_streaming_attn_fwd`
+// (src/streaming_attention/kernel.py:196-430).  One workgroup owns TQ = 32*NW queries of
+// one (batch, head); each wave owns 32 of them and each lane one query column, so the
+// running max / sum and the [lo, hi) key window of a query are per-lane scalars.
+// The workgroup visits only the key tiles that intersect the window of its queries
+// (kernel.py:282-291); tiles that lie wholly inside every lane's window skip the mask.
+#pragma once
+#include "sa_common.h"
+
+namespace sa {
+
+template <typename T, int D, int NW, int TK>
+__global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
+  using E = Elem<T>;
+  using G = TileGeom<T, D>;
+  using Frag = typename E::Frag;
+  constexpr int TQ = NW * 32, NT = NW * 64, KBN = TK / 32;
+  constexpr int PITCH = G::PITCH, NF = G::NF, DB = G::DB;
+  constexpr int TILE = TK * PITCH;  // elements per staged K or V tile
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  T* smem = reinterpret_cast<T*>(smem_raw);  // [stage][K|V][TK][PITCH]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int bid = xcd_remap(blockIdx.x, gridDim.x);
+  const int qt = bid % p.n_tiles;
+  const int bh = bid / p.n_tiles;
+  const int hd = bh % p.H, b = bh / p.H;
+  const int T_ = p.T, C = p.C, R = p.R;
+
+  int L = T_;
+  if (p.lens) {
+    L = p.lens[(int64_t)b * p.lens_stride];
+    L = L < 0 ? 0 : (L > T_ ? T_ : L);
+  }
+  const int q0 = qt * TQ;
+  T* o_base = reinterpret_cast<T*>(p.o) + (int64_t)bh * T_ * D;
+  float* lse_base = p.lse ? p.lse + (int64_t)bh * T_ : nullptr;
+  const int q_end = q0 + TQ < T_ ? q0 + TQ : T_;
+
+  if (q0 >= L) {  // whole tile is padding: the outputs there are defined as zero
+    zero_rows<T, D, NT>(o_base, q0, q_end, tid);
+    if (lse_base)
+      for (int r = q0 + tid; r < q_end; r += NT) lse_base[r] = 0.0f;
+    return;
+  }
+
+  // ---- per-lane query and its key window ------------------------------------------
+  const int qrow = q0 + wave * 32 + c;
+  const int qe = qrow < L ? qrow : L - 1;  // rows past L mimic the last valid row
+  const int qchunk = qe / C;
+  const int lo = (qchunk > R ? qchunk - R : 0) * C;
+  const int hi = (qchunk + 1) * C < L ? (qchunk + 1) * C : L;
+  // the tightest window over the wave decides whether a tile needs masking at all
+  const int wq_first = q0 + wave * 32 < L ? q0 + wave * 32 : L - 1;
+  const int wq_last = q0 + wave * 32 + 31 < L ? q0 + wave * 32 + 31 : L - 1;
+  const int hi_min = (wq_first / C + 1) * C < L ? (wq_first / C + 1) * C : L;
+  const int lo_max = (wq_last / C > R ? wq_last / C - R : 0) * C;
+  // union over the workgroup decides which tiles are visited
+  const int gq_last = q0 + TQ - 1 < L ? q0 + TQ - 1 : L - 1;
+  const int lo_wg = (q0 / C > R ? q0 / C - R : 0) * C;
+  const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
+  const int kt0 = lo_wg / TK, kt1 = (hi_wg + TK - 1) / TK;
+
+  const float sl2e = fabsf(p.scale_log2e);
+  const bool neg = p.scale_log2e < 0.0f;
+
+  // ---- Q fragments stay in registers for the whole key loop -------------------------
+  Frag qf[NF];
+  {
+    const int qr = qrow < T_ ? qrow : T_ - 1;
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh +
+                  (int64_t)qr * p.q_st;
+#pragma unroll
+    for (int g = 0; g < NF; ++g) {
+      qf[g] = *reinterpret_cast<const Frag*>(qp + (g * 2 + h) * E::VEC);
+      if (neg) qf[g] = negate<T>(qf[g]);
+    }
+  }
+
+  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh;
+  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh;
+
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int m = 0; m < DB; ++m)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[m][i] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  Stager<T, D, TK, NT> sk, sv;
+  sk.load(kbase, p.k_st, kt0 * TK, T_ - 1, tid);
+  sv.load(vbase, p.v_st, kt0 * TK, T_ - 1, tid);
+  sk.store(smem, tid);
+  sv.store(smem + TILE, tid);
+  __syncthreads();
+
+  for (int t = kt0; t < kt1; ++t) {
+    const int cur = (t - kt0) & 1;
+    const T* Kt = smem + cur * 2 * TILE;
+    const T* Vt = Kt + TILE;
+    const bool more = t + 1 < kt1;
+    if (more) {
+      sk.load(kbase, p.k_st, (t + 1) * TK, T_ - 1, tid);
+      sv.load(vbase, p.v_st, (t + 1) * TK, T_ - 1, tid);
+    }
+    const int k0 = t * TK;
+
+    // S^T[key][q] = K Q^T
+    f32x16 s[KBN];
+#pragma unroll
+    for (int kb = 0; kb < KBN; ++kb) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[kb][i] = 0.0f;
+#pragma unroll
+      for (int g = 0; g < NF; ++g) mma(s[kb], lds_row_frag<T, PITCH>(Kt, kb * 32 + c, g, h), qf[g]);
+    }
+
+#pragma unroll
+    for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[kb][i] *= sl2e;
+
+    const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
+    if (!interior) {
+#pragma unroll
+      for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = k0 + kb * 32 + crow(i, h);
+          if (key < lo || key >= hi) s[kb][i] = -INFINITY;
+        }
+    }
+
+    // online softmax in base 2; the two halves of the wave hold disjoint keys of
+    // the same query, so only the max has to cross lanes inside the loop
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
+    mx = half_max(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);
+    float rs = 0.0f;
+#pragma unroll
+    for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float e = fast_exp2(s[kb][i] - m_safe);
+        s[kb][i] = e;
+        rs += e;
+      }
+    l_run = l_run * alpha + rs;
+    m_run = m_new;
+#pragma unroll
+    for (int m = 0; m < DB; ++m)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[m][i] *= alpha;
+
+    // O^T[d][q] += V^T P^T
+#pragma unroll
+    for (int kb = 0; kb < KBN; ++kb) mma_tr<T, PITCH, DB>(oacc, Vt, kb, s[kb], lane);
+
+    if (more) {
+      T* nxt = smem + (cur ^ 1) * 2 * TILE;
+      sk.store(nxt, tid);
+      sv.store(nxt + TILE, tid);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue --------------------------------------------------------------------
+  const float l_tot = half_sum(l_run);
+  const bool valid = qrow < L;
+  if (qrow < T_) {
+    const float inv = valid ? 1.0f / l_tot : 0.0f;
+    if (!valid) {
+#pragma unroll
+      for (int m = 0; m < DB; ++m)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[m][i] = 0.0f;
+    }
+    store_acc_T<T, D, DB>(o_base + (int64_t)qrow * D, oacc, inv, h);
+    if (lse_base && h == 0) lse_base[qrow] = valid ? m_run + __builtin_amdgcn_logf(l_tot) : 0.0f;
+  }
+}
+
+}  // namespace sa

@@ -1,0 +1,119 @@
+// Kernel instantiations for one element type and one kernel family.
+// Compiled once per (SA_DTYPE_ID, SA_KIND) pair so that the families build in parallel.
+//   SA_DTYPE_ID: 0 fp32, 1 fp16, 2 bf16        SA_KIND: 0 forward, 1 delta + dQ, 2 dK/dV
+#include <mutex>
+#include "sa_launch.h"
+#if SA_KIND == 0
+#include "sa_fwd.h"
+#else
+#include "sa_bwd.h"
+#endif
+
+namespace sa {
+
+#if SA_DTYPE_ID == 0
+using ElemT = float;
+#elif SA_DTYPE_ID == 1
+using ElemT = _Float16;
+#elif SA_DTYPE_ID == 2
+using ElemT = __bf16;
+#else
+#error "SA_DTYPE_ID must be 0, 1 or 2"
+#endif
+
+template <typename K> static int prepare(K kernel, size_t lds_bytes, std::once_flag& once) {
+  int rc = 0;
+  std::call_once(once, [&] {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    rc = (int)e;
+  });
+  return rc;
+}
+
+static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+#define SA_FOR_EACH_D(X) \
+  switch (D) {           \
+    case 16: X(16);      \
+    case 32: X(32);      \
+    case 64: X(64);      \
+    case 128: X(128);    \
+    case 256: X(256);    \
+    default: return SA_ERR_HEAD_DIM; \
+  }
+
+#if SA_KIND == 0
+template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
+  using C = Cfg<ElemT>;
+  constexpr int TQ = C::NW * 32;
+  constexpr size_t lds = (size_t)2 * 2 * C::FWD_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
+  auto kern = fwd_kernel<ElemT, D, C::NW, C::FWD_TK>;
+  static std::once_flag once;
+  if (int rc = prepare(kern, lds, once)) return rc;
+  p.n_tiles = (int)ceil_div(p.T, TQ);
+  const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+  if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
+  return (int)hipGetLastError();
+}
+template <> int launch_fwd<ElemT>(const FwdParams& p, int D, hipStream_t st) {
+#define X(d) return fwd_d<d>(p, st)
+  SA_FOR_EACH_D(X)
+#undef X
+}
+#elif SA_KIND == 1
+template <int D> static int delta_d(const DeltaParams& p, hipStream_t st) {
+  constexpr int RPB = 256 / (D / Elem<ElemT>::VEC);
+  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  const int64_t blocks = ceil_div(rows, RPB);
+  if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+  hipLaunchKernelGGL((delta_kernel<ElemT, D>), dim3((unsigned)blocks), dim3(256), 0, st, p);
+  return (int)hipGetLastError();
+}
+template <> int launch_delta<ElemT>(const DeltaParams& p, int D, hipStream_t st) {
+#define X(d) return delta_d<d>(p, st)
+  SA_FOR_EACH_D(X)
+#undef X
+}
+template <int D> static int dq_d(BwdParams p, hipStream_t st) {
+  using C = Cfg<ElemT>;
+  constexpr int TQ = C::NW * 32;
+  constexpr size_t lds = (size_t)2 * 2 * C::DQ_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
+  auto kern = dq_kernel<ElemT, D, C::NW, C::DQ_TK>;
+  static std::once_flag once;
+  if (int rc = prepare(kern, lds, once)) return rc;
+  p.n_tiles = (int)ceil_div(p.T, TQ);
+  const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+  if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
+  return (int)hipGetLastError();
+}
+template <> int launch_dq<ElemT>(const BwdParams& p, int D, hipStream_t st) {
+#define X(d) return dq_d<d>(p, st)
+  SA_FOR_EACH_D(X)
+#undef X
+}
+#else
+template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
+  using C = Cfg<ElemT>;
+  constexpr int TKB = C::NW * 32;
+  constexpr size_t lds =
+      (size_t)2 * (2 * C::DKDV_TQ * TileGeom<ElemT, D>::PITCH * sizeof(ElemT) + 2 * C::DKDV_TQ * sizeof(float));
+  auto kern = dkdv_kernel<ElemT, D, C::NW, C::DKDV_TQ>;
+  static std::once_flag once;
+  if (int rc = prepare(kern, lds, once)) return rc;
+  p.n_tiles = (int)ceil_div(p.T, TKB);
+  const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+  if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
+  return (int)hipGetLastError();
+}
+template <> int launch_dkdv<ElemT>(const BwdParams& p, int D, hipStream_t st) {
+#define X(d) return dkdv_d<d>(p, st)
+  SA_FOR_EACH_D(X)
+#undef X
+}
+#endif
+
+}  // namespace sa

@@ -1,0 +1,213 @@
+"""The operator boundary: ``alexdremov_streaming_attention::forward`` / ``::backward``.
+
+Same dispatcher names, argument lists, fake implementations and autograd registration as
+the reference (src/streaming_attention/kernel.py:1270-1530); the bodies enqueue the HIP
+kernels of libstreaming_attention.so on the current stream instead of launching Triton
+kernels.  ``autotune``, ``prescale_qk`` and ``precision`` are accepted for signature
+compatibility and do not change the result: tile shapes are fixed per (dtype, head_dim)
+and all accumulation is fp32.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_HEAD_DIMS = (16, 32, 64, 128, 256)
+_VEC_BYTES = 16
+
+
+def _dtype_id(dtype: torch.dtype) -> int:
+    try:
+        return _lib.DTYPE_IDS[str(dtype)]
+    except KeyError:
+        raise AssertionError(f"unsupported dtype {dtype}: expected float32, float16 or bfloat16") from None
+
+
+def _kernel_layout(t: torch.Tensor) -> torch.Tensor:
+    """Return ``t`` itself when the kernels can read it in place (unit stride along the head
+    dimension, every other stride and the base address a multiple of 16 bytes), otherwise a
+    contiguous copy."""
+    es = t.element_size()
+    vec = _VEC_BYTES // es
+    ok = (
+        t.stride(-1) == 1
+        and all(s % vec == 0 for s in t.stride()[:-1])
+        and t.data_ptr() % _VEC_BYTES == 0
+    )
+    return t if ok else t.contiguous()
+
+
+def _lens_args(lens: Optional[torch.Tensor]):
+    if lens is None:
+        return None, 0
+    return lens.data_ptr(), lens.stride(0)
+
+
+def _stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _validate(q, k, v, lens, context_size, back_contexts, sm_scale):
+    # same conditions, same exception type as kernel.py:1288-1295
+    batch, _, T, head_dim = q.shape
+    assert back_contexts >= 0 and context_size >= 1
+    assert head_dim in _HEAD_DIMS
+    assert head_dim == k.shape[-1] and head_dim == v.shape[-1]
+    assert T == k.shape[-2] and T == v.shape[-2]
+    assert sm_scale is not None
+    assert lens is None or (lens.dtype == torch.int32 and batch == len(lens) and lens.ndim == 1)
+    assert q.dtype == k.dtype == v.dtype
+
+
+@torch.library.custom_op(
+    "alexdremov_streaming_attention::forward", mutates_args=(), device_types=("cuda",)
+)
+def attention_forward_adapter(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    lens: Optional[torch.Tensor],
+    context_size: int,
+    back_contexts: int,
+    sm_scale: float,
+    autotune: bool,
+    return_lse: bool,
+    prescale_qk: bool,
+    precision: str,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    _validate(q, k, v, lens, context_size, back_contexts, sm_scale)
+    B, H, T, D = q.shape
+    lib = _lib.load()
+    # the kernel writes every element (zeros at padded positions included)
+    O = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    LSE = torch.empty((B, H, T), dtype=torch.float32, device=q.device) if return_lse else None
+    if q.numel() > 0:
+        qk, kk, vk = _kernel_layout(q), _kernel_layout(k), _kernel_layout(v)
+        lens_ptr, lens_stride = _lens_args(lens)
+        with torch.cuda.device(q.device):
+            rc = lib.sa_forward(
+                qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), lens_ptr, lens_stride,
+                O.data_ptr(), LSE.data_ptr() if LSE is not None else None,
+                _lib.strides4(qk), _lib.strides4(kk), _lib.strides4(vk),
+                B, H, T, D, min(int(context_size), 2**31 - 1), min(int(back_contexts), 2**31 - 1),
+                float(sm_scale), _dtype_id(q.dtype), _stream(q.device),
+            )
+        _lib.check(rc, "sa_forward")
+    if LSE is None:
+        LSE = torch.empty(0)
+    return O, LSE
+
+
+@torch.library.register_fake("alexdremov_streaming_attention::forward")
+def attention_forward_adapter_abstract(
+    q, k, v, lens, context_size, back_contexts, sm_scale, autotune, return_lse, prescale_qk, precision
+):
+    return (
+        torch.empty_like(q, memory_format=torch.contiguous_format),
+        torch.empty(q.shape[:3], dtype=torch.float32, device=q.device) if return_lse else torch.empty(0),
+    )
+
+
+@torch.library.custom_op(
+    "alexdremov_streaming_attention::backward", mutates_args=(), device_types=("cuda",)
+)
+def attention_backward_adapter(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    lens: Optional[torch.Tensor],
+    o: torch.Tensor,
+    lse: torch.Tensor,
+    do: torch.Tensor,
+    context_size: int,
+    back_contexts: int,
+    sm_scale: float,
+    autotune: bool,
+    prescale_qk: bool,
+    precision: str,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _validate(q, k, v, lens, context_size, back_contexts, sm_scale)
+    B, H, T, D = q.shape
+    lib = _lib.load()
+    DQ = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    DK = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    DV = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+    if q.numel() == 0:
+        return DQ, DK, DV
+    qk, kk, vk = _kernel_layout(q), _kernel_layout(k), _kernel_layout(v)
+    # the upstream gradient may arrive in another dtype and with arbitrary strides
+    # (tests/test_streaming_attention.py:224-248 hands an fp32 strided one to fp16 q/k/v)
+    gk = _kernel_layout(do if do.dtype == q.dtype else do.to(q.dtype))
+    ok = _kernel_layout(o if o.dtype == q.dtype else o.to(q.dtype))
+    lens_ptr, lens_stride = _lens_args(lens)
+    dt = _dtype_id(q.dtype)
+    C = min(int(context_size), 2**31 - 1)
+    R = min(int(back_contexts), 2**31 - 1)
+    with torch.cuda.device(q.device):
+        stream = _stream(q.device)
+        if lse.numel() != B * H * T or lse.device != q.device:
+            # forward was run with return_lse=False: rebuild the log-sum-exp
+            lse = torch.empty((B, H, T), dtype=torch.float32, device=q.device)
+            scratch = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+            rc = lib.sa_forward(
+                qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), lens_ptr, lens_stride,
+                scratch.data_ptr(), lse.data_ptr(),
+                _lib.strides4(qk), _lib.strides4(kk), _lib.strides4(vk),
+                B, H, T, D, C, R, float(sm_scale), dt, stream,
+            )
+            _lib.check(rc, "sa_forward (log-sum-exp rebuild)")
+        lse = lse.contiguous()
+        if lse.dtype != torch.float32:
+            lse = lse.float()
+        delta = torch.empty((B, H, T), dtype=torch.float32, device=q.device)
+        rc = lib.sa_backward(
+            qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), lens_ptr, lens_stride,
+            ok.data_ptr(), gk.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            DQ.data_ptr(), DK.data_ptr(), DV.data_ptr(),
+            _lib.strides4(qk), _lib.strides4(kk), _lib.strides4(vk), _lib.strides4(ok), _lib.strides4(gk),
+            B, H, T, D, C, R, float(sm_scale), dt, stream,
+        )
+    _lib.check(rc, "sa_backward")
+    return DQ, DK, DV
+
+
+@torch.library.register_fake("alexdremov_streaming_attention::backward")
+def attention_backward_adapter_abstract(
+    q, k, v, lens, o, lse, do, context_size, back_contexts, sm_scale, autotune, prescale_qk, precision
+):
+    return (
+        torch.empty_like(q, memory_format=torch.contiguous_format),
+        torch.empty_like(k, memory_format=torch.contiguous_format),
+        torch.empty_like(v, memory_format=torch.contiguous_format),
+    )
+
+
+def _setup_context(ctx, inputs, output):
+    O, LSE = output
+    (q, k, v, lens, context_size, back_contexts, sm_scale, autotune, return_lse, prescale_qk, precision) = inputs
+    ctx.save_for_backward(q, k, v, O, LSE, lens)
+    ctx.context_size = context_size
+    ctx.back_contexts = back_contexts
+    ctx.autotune = autotune
+    ctx.sm_scale = sm_scale
+    ctx.prescale_qk = prescale_qk
+    ctx.precision = precision
+
+
+def _backward(ctx, do, dlse):
+    # no gradient flows through the log-sum-exp output (kernel.py:1498)
+    q, k, v, o, lse, lens = ctx.saved_tensors
+    DQ, DK, DV = torch.ops.alexdremov_streaming_attention.backward(
+        q=q, k=k, v=v, lens=lens, o=o, lse=lse, do=do,
+        context_size=ctx.context_size, back_contexts=ctx.back_contexts, sm_scale=ctx.sm_scale,
+        autotune=ctx.autotune, prescale_qk=ctx.prescale_qk, precision=ctx.precision,
+    )
+    return DQ, DK, DV, None, None, None, None, None, None, None, None
+
+
+torch.library.register_autograd(
+    "alexdremov_streaming_attention::forward", _backward, setup_context=_setup_context
+)
