@@ -1,0 +1,229 @@
+#!/usr/bin/env python3
+"""Benchmark of the streaming-attention hot path on one MI355X.
+
+A step is one forward + backward of the operator through its public API on one batch of
+synthetic inputs already resident in HBM.  The headline workload is
+B=4, H=16, T=16384, D=128, bf16, chunk 256, 8 back chunks, lens ~ U{T/2..T}.
+
+Prints one JSON line:
+  value      effective TFLOP/s = 14*D*H*P / step time, P = unmasked (query, key) pairs
+  roofline   the dominant kernel (longest average launch) timed on its own with HIP events
+             on the launch stream, against the dense bf16 MFMA peak
+  cpu_baseline  the masked-SDPA oracle (the reference's torch formulation) forward+backward
+             in fp32 on the host cores, on a bounded sample
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "kernels_amd"))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
+
+WORKLOADS = {
+    # name: (B, H, T, D, dtype, C, R, lens mode, q/k/v scale)
+    "cpu_ref_fp32": (2, 4, 512, 64, "float32", 64, 2, "uniform_256_512", 1.0),
+    "bf16_T4096_D64": (8, 16, 4096, 64, "bfloat16", 128, 4, "full", None),
+    "headline_bf16_T16384_D128": (4, 16, 16384, 128, "bfloat16", 256, 8, "uniform_half_full", 1.0),
+    "ragged_fp16_T2048_D128": (16, 8, 2048, 128, "float16", 64, 1, "loguniform_64_T", 1.0),
+    "long_bf16_T65536_D128": (1, 32, 65536, 128, "bfloat16", 512, 16, "full", 1.0),
+}
+DEFAULT = "headline_bf16_T16384_D128"
+
+
+def unmasked_pairs(T, C, R, lens_list):
+    """Allowed (query, key) pairs per head, summed over the batch (closed form per chunk)."""
+    total = 0
+    for L in lens_list:
+        L = min(int(L), T)
+        c = 0
+        while c * C < L:
+            rows = min((c + 1) * C, L) - c * C
+            keys = min((c + 1) * C, L) - max(0, c - R) * C
+            total += rows * keys
+            c += 1
+    return total
+
+
+def make_inputs(name, device):
+    import torch
+
+    B, H, T, D, dtype_name, C, R, lens_mode, qkv_scale = WORKLOADS[name]
+    dtype = getattr(torch, dtype_name)
+    g = torch.Generator().manual_seed(20)
+    if lens_mode == "full":
+        lens = None
+        lens_list = [T] * B
+    elif lens_mode == "uniform_half_full":
+        lens = torch.randint(T // 2, T + 1, (B,), generator=g, dtype=torch.int32)
+    elif lens_mode == "uniform_256_512":
+        lens = torch.randint(256, 513, (B,), generator=g, dtype=torch.int32)
+    elif lens_mode == "loguniform_64_T":
+        u = torch.rand(B, generator=g, dtype=torch.float64)
+        lens = torch.exp(math.log(64.0) + u * (math.log(T) - math.log(64.0))).round().to(torch.int32)
+    else:
+        raise ValueError(lens_mode)
+    if lens is not None:
+        lens_list = lens.tolist()
+    dg = torch.Generator(device=device).manual_seed(20)
+    scale = D ** -0.5 if qkv_scale is None else qkv_scale
+    q, k, v = [(torch.randn(B, H, T, D, generator=dg, device=device, dtype=torch.float32) * scale).to(dtype)
+               for _ in range(3)]
+    d_o = torch.randn(B, H, T, D, generator=dg, device=device, dtype=torch.float32).to(dtype)
+    return dict(q=q, k=k, v=v, d_o=d_o, lens=lens.to(device) if lens is not None else None,
+                lens_list=lens_list, B=B, H=H, T=T, D=D, C=C, R=R, dtype=dtype_name)
+
+
+def time_kernels(w, iters):
+    """Average duration of each kernel launched on its own through the C ABI, in ms."""
+    import torch
+    from streaming_attention import _lib
+
+    lib = _lib.load()
+    q, k, v, d_o, lens = w["q"], w["k"], w["v"], w["d_o"], w["lens"]
+    B, H, T, D, C, R = w["B"], w["H"], w["T"], w["D"], w["C"], w["R"]
+    dt = _lib.DTYPE_IDS["torch." + w["dtype"]]
+    scale = D ** -0.5
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, T, dtype=torch.float32, device=q.device)
+    delta = torch.empty_like(lse)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    lp, ls = (lens.data_ptr(), lens.stride(0)) if lens is not None else (None, 0)
+    st = torch.cuda.current_stream().cuda_stream
+    s4 = _lib.strides4
+
+    def fwd():
+        return lib.sa_forward(q.data_ptr(), k.data_ptr(), v.data_ptr(), lp, ls, o.data_ptr(), lse.data_ptr(),
+                              s4(q), s4(k), s4(v), B, H, T, D, C, R, scale, dt, st)
+
+    def dlt():
+        return lib.sa_bwd_delta(o.data_ptr(), d_o.data_ptr(), delta.data_ptr(), s4(o), s4(d_o), B, H, T, D, dt, st)
+
+    def dqf():
+        return lib.sa_bwd_dq(q.data_ptr(), k.data_ptr(), v.data_ptr(), lp, ls, d_o.data_ptr(), lse.data_ptr(),
+                             delta.data_ptr(), dq.data_ptr(), s4(q), s4(k), s4(v), s4(d_o),
+                             B, H, T, D, C, R, scale, dt, st)
+
+    def dkv():
+        return lib.sa_bwd_dkdv(q.data_ptr(), k.data_ptr(), v.data_ptr(), lp, ls, d_o.data_ptr(), lse.data_ptr(),
+                               delta.data_ptr(), dk.data_ptr(), dv.data_ptr(), s4(q), s4(k), s4(v), s4(d_o),
+                               B, H, T, D, C, R, scale, dt, st)
+
+    out = {}
+    for name, fn in (("fwd", fwd), ("delta", dlt), ("dq", dqf), ("dkdv", dkv)):
+        _lib.check(fn(), name)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()   # events and launches share torch's current stream `st`
+        for _ in range(iters):
+            fn()
+        e1.record()
+        e1.synchronize()
+        out[name] = e0.elapsed_time(e1) / iters
+    return out
+
+
+def cpu_baseline(max_seconds=20.0):
+    """Masked-SDPA oracle forward+backward, fp32, on the host cores (config 1 of the baseline)."""
+    import torch
+    from oracle import sa_oracle
+
+    B, H, T, D, _, C, R, _, _ = WORKLOADS["cpu_ref_fp32"]
+    g = torch.Generator().manual_seed(20)
+    q, k, v, d_o = [torch.randn(B, H, T, D, generator=g) for _ in range(4)]
+    lens = torch.randint(256, 513, (B,), generator=g, dtype=torch.int32)
+    P = unmasked_pairs(T, C, R, lens.tolist())
+    flops = 14.0 * D * H * P
+    for _ in range(3):
+        sa_oracle.sdpa_fwd_bwd(q, k, v, lens, C, R, d_o)
+    n, t0 = 0, time.perf_counter()
+    while n < 10 or (time.perf_counter() - t0 < 2.0 and n < 1000):
+        sa_oracle.sdpa_fwd_bwd(q, k, v, lens, C, R, d_o)
+        n += 1
+        if time.perf_counter() - t0 > max_seconds:
+            break
+    dt = (time.perf_counter() - t0) / n
+    return {
+        "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"B={B} H={H} T={T} D={D} fp32 chunk={C} back={R} lens~U[256,512], {n} fwd+bwd iterations "
+                  f"of the dense-mask SDPA oracle, {dt * 1e3:.2f} ms each, host has {os.cpu_count()} logical cpus",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernel-iters", type=int, default=10)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+
+    import torch
+    from streaming_attention import streaming_attention
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    w = make_inputs(args.workload, dev)
+    B, H, T, D, C, R = w["B"], w["H"], w["T"], w["D"], w["C"], w["R"]
+    P = unmasked_pairs(T, C, R, w["lens_list"])
+    flops_step = 14.0 * D * H * P
+    q, k, v = (w[n].requires_grad_() for n in ("q", "k", "v"))
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        out = streaming_attention(q, k, v, w["lens"], C, R)
+        out.backward(w["d_o"])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = flops_step / (ms_per_step * 1e-3) / 1e12
+
+    kt = time_kernels(w, args.kernel_iters)
+    # GEMMs each kernel performs per unmasked pair: fwd S,PV; dq S,dP,dQ; dkdv S,dP,dV,dK
+    kernel_flops = {"fwd": 4.0 * D * H * P, "dq": 6.0 * D * H * P, "dkdv": 8.0 * D * H * P}
+    dom = max(kernel_flops, key=lambda n: kt[n])
+    achieved = kernel_flops[dom] / (kt[dom] * 1e-3) / 1e12
+    es = 4 if w["dtype"] == "float32" else 2
+    N = B * H * T
+    result = {
+        "metric": "effective TFLOP/s fwd+bwd (unmasked blocks) at 1 GPU; % of bf16 MFMA peak",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"bfloat16": "bf16", "float16": "f16", "float32": "f32"}[w["dtype"]],
+        "data": "synthetic",
+        "config": {"workload": args.workload, "B": B, "H": H, "T": T, "D": D, "context_size": C,
+                   "back_contexts": R, "lens": w["lens_list"], "unmasked_pairs_per_head": P,
+                   "flops_per_step": flops_step},
+        "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
+        "peaks_used": {"bf16_mfma_tflops": PEAK_BF16_TFLOPS, "hbm_gbs": PEAK_HBM_GBS},
+        "kernel_ms": kt,
+        "kernel_tflops": {n: kernel_flops[n] / (kt[n] * 1e-3) / 1e12 for n in kernel_flops},
+        "delta_gbs": (2.0 * N * D * es + 4.0 * N) / (kt["delta"] * 1e-3) / 1e9,
+        "roofline": {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

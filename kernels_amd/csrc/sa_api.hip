@@ -66,7 +66,9 @@ int sa_forward(const void* q, const void* k, const void* v, const int32_t* lens,
   p.B = B; p.H = H; p.T = T; p.C = context_size; p.R = back_contexts;
   clamp_window(T, p.C, p.R);
   p.scale_log2e = sm_scale * kLog2e;
-  return by_dtype(dtype, [&](auto tag) { return launch_fwd<decltype(tag)>(p, D, (hipStream_t)stream); });
+  return by_dtype(dtype, [&](auto tag) {
+    using E = decltype(tag);
+    return D == 256 ? launch_fwd<E, 1>(p, D, (hipStream_t)stream) : launch_fwd<E, 0>(p, D, (hipStream_t)stream); });
 }
 
 int sa_bwd_delta(const void* o, const void* d_o, float* delta, const int64_t* os, const int64_t* gs, int B,
@@ -81,7 +83,9 @@ int sa_bwd_delta(const void* o, const void* d_o, float* delta, const int64_t* os
   p.o_sb = os[0]; p.o_sh = os[1]; p.o_st = os[2];
   p.do_sb = gs[0]; p.do_sh = gs[1]; p.do_st = gs[2];
   p.B = B; p.H = H; p.T = T;
-  return by_dtype(dtype, [&](auto tag) { return launch_delta<decltype(tag)>(p, D, (hipStream_t)stream); });
+  return by_dtype(dtype, [&](auto tag) {
+    using E = decltype(tag);
+    return D == 256 ? launch_delta<E, 1>(p, D, (hipStream_t)stream) : launch_delta<E, 0>(p, D, (hipStream_t)stream); });
 }
 
 static int fill_bwd(BwdParams& p, const void* q, const void* k, const void* v, const int32_t* lens,
@@ -120,7 +124,9 @@ int sa_bwd_dq(const void* q, const void* k, const void* v, const int32_t* lens, 
   if (B == 0 || H == 0 || T == 0) return SA_OK;
   if (!dq || !aligned16(dq)) return dq ? SA_ERR_LAYOUT : SA_ERR_ARG;
   p.dq = dq;
-  return by_dtype(dtype, [&](auto tag) { return launch_dq<decltype(tag)>(p, D, (hipStream_t)stream); });
+  return by_dtype(dtype, [&](auto tag) {
+    using E = decltype(tag);
+    return D == 256 ? launch_dq<E, 1>(p, D, (hipStream_t)stream) : launch_dq<E, 0>(p, D, (hipStream_t)stream); });
 }
 
 int sa_bwd_dkdv(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
@@ -135,7 +141,9 @@ int sa_bwd_dkdv(const void* q, const void* k, const void* v, const int32_t* lens
   if (!dk || !dv) return SA_ERR_ARG;
   if (!aligned16(dk) || !aligned16(dv)) return SA_ERR_LAYOUT;
   p.dk = dk; p.dv = dv;
-  return by_dtype(dtype, [&](auto tag) { return launch_dkdv<decltype(tag)>(p, D, (hipStream_t)stream); });
+  return by_dtype(dtype, [&](auto tag) {
+    using E = decltype(tag);
+    return D == 256 ? launch_dkdv<E, 1>(p, D, (hipStream_t)stream) : launch_dkdv<E, 0>(p, D, (hipStream_t)stream); });
 }
 
 int sa_backward(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,

@@ -131,6 +131,7 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(const BwdParams p) {
   sv.load(vbase, p.v_st, kt0 * TK, T_ - 1, tid);
   sk.store(smem, tid);
   sv.store(smem + TILE, tid);
+  wait_all_loads();
   __syncthreads();
 
   for (int t = kt0; t < kt1; ++t) {
@@ -150,22 +151,26 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(const BwdParams p) {
       f32x16 s, dp;
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[i] = 0.0f, dp[i] = 0.0f;
-#pragma unroll
-      for (int g = 0; g < NF; ++g) mma(s, lds_row_frag<T, PITCH>(Kt, kb * 32 + c, g, h), qf[g]);
-#pragma unroll
-      for (int g = 0; g < NF; ++g) mma(dp, lds_row_frag<T, PITCH>(Vt, kb * 32 + c, g, h), gf[g]);
+      {
+        f32x16 (&s1)[1] = reinterpret_cast<f32x16(&)[1]>(s);
+        f32x16 (&dp1)[1] = reinterpret_cast<f32x16(&)[1]>(dp);
+        mma_rows<T, D>(s1, Kt, kb * 32, qf, lane);
+        mma_rows<T, D>(dp1, Vt, kb * 32, gf, lane);
+      }
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        float pr = fast_exp2(s[i] * sl2e - lse_q);
-        float ds = pr * (dp[i] - delta_q);
-        if (!interior) {
+        const float pr = fast_exp2(s[i] * sl2e - lse_q);
+        s[i] = pr * (dp[i] - delta_q);
+      }
+      if (!interior) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
           const int key = k0 + kb * 32 + crow(i, h);
-          if (key < lo || key >= hi) ds = 0.0f;
+          s[i] = (key < lo || key >= hi) ? 0.0f : s[i];
         }
-        s[i] = ds;
       }
       // dQ^T[d][q] += K^T dS^T
-      mma_tr<T, PITCH, DB>(acc, Kt, kb, s, lane);
+      mma_tr<T, D>(acc, Kt, kb, s, lane);
     }
 
     if (more) {
@@ -296,6 +301,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   sg.load(gbase, p.do_st, qt0 * TQ, T_ - 1, tid);
   load_rows(qt0 * TQ);
   store_stage(0);
+  wait_all_loads();
   __syncthreads();
 
   for (int t = qt0; t < qt1; ++t) {
@@ -319,10 +325,12 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[i] = 0.0f, dp[i] = 0.0f;
       // S[q][key] = Q K^T, dP[q][key] = dO V^T
-#pragma unroll
-      for (int g = 0; g < NF; ++g) mma(s, lds_row_frag<T, PITCH>(Qt, qb * 32 + c, g, h), kf[g]);
-#pragma unroll
-      for (int g = 0; g < NF; ++g) mma(dp, lds_row_frag<T, PITCH>(Gt, qb * 32 + c, g, h), vf[g]);
+      {
+        f32x16 (&s1)[1] = reinterpret_cast<f32x16(&)[1]>(s);
+        f32x16 (&dp1)[1] = reinterpret_cast<f32x16(&)[1]>(dp);
+        mma_rows<T, D>(s1, Qt, qb * 32, kf, lane);
+        mma_rows<T, D>(dp1, Gt, qb * 32, vf, lane);
+      }
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_t + qb * 32 + 8 * g4 + 4 * h);
@@ -330,21 +338,23 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int i = 4 * g4 + e;
-          float pr = fast_exp2(s[i] * sl2e - l4[e]);
-          float ds = pr * (dp[i] - d4[e]);
-          if (!interior) {
-            const int qr = qs + qb * 32 + crow(i, h);
-            const bool ok = qr >= qlo && qr < qhi;
-            pr = ok ? pr : 0.0f;
-            ds = ok ? ds : 0.0f;
-          }
+          const float pr = fast_exp2(s[i] * sl2e - l4[e]);
           s[i] = pr;
-          dp[i] = ds;
+          dp[i] = pr * (dp[i] - d4[e]);
+        }
+      }
+      if (!interior) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int qr = qs + qb * 32 + crow(i, h);
+          const bool ok = qr >= qlo && qr < qhi;
+          s[i] = ok ? s[i] : 0.0f;
+          dp[i] = ok ? dp[i] : 0.0f;
         }
       }
       // dV^T[d][key] += dO^T P,  dK^T[d][key] += Q^T dS
-      mma_tr<T, PITCH, DB>(dv, Gt, qb, s, lane);
-      mma_tr<T, PITCH, DB>(dk, Qt, qb, dp, lane);
+      mma_tr<T, D>(dv, Gt, qb, s, lane);
+      mma_tr<T, D>(dk, Qt, qb, dp, lane);
     }
 
     if (more) store_stage(cur ^ 1);

@@ -62,13 +62,40 @@ template <> struct Elem<float> {
   static constexpr uint32_t SIGN = 0x80000000u;
 };
 
-// LDS row pitch in elements: the head dimension (at least one 32-wide block, so that
-// transposed reads of a D=16 tile stay inside the row) plus one 16-byte pad.
+// LDS tile geometry.  Two layouts:
+//  * swizzled (16-bit types, D >= 64): rows are stored unpadded and the 16-byte chunk index
+//    inside a row is XOR-ed with a permutation of the low row bits, chosen so that both access
+//    patterns of the kernels spread over all 64 banks: 16 lanes reading the same chunk of 16
+//    consecutive rows (row-major fragments), and 32 lanes reading a 4-row x 64-byte patch
+//    (transposing reads).
+//  * padded (everything else): the head dimension (at least one 32-wide block, so that
+//    transposed reads of a D=16 tile stay inside the row) plus one 16-byte pad.
+#ifndef SA_PAD_VECS
+#define SA_PAD_VECS 1
+#endif
+#ifndef SA_SWIZZLE
+#define SA_SWIZZLE 1
+#endif
 template <typename T, int D> struct TileGeom {
+  static constexpr int VEC = Elem<T>::VEC;
   static constexpr int DP = D < 32 ? 32 : D;
-  static constexpr int PITCH = DP + Elem<T>::VEC;
-  static constexpr int NF = D / (2 * Elem<T>::VEC);   // row fragments per lane
-  static constexpr int DB = DP / 32;                  // 32-wide blocks along D
+  static constexpr bool SWZ = SA_SWIZZLE && Elem<T>::HALF && D >= 64;
+  static constexpr int PITCH = SWZ ? D : DP + SA_PAD_VECS * VEC;
+  static constexpr int NF = D / (2 * VEC);   // row fragments per lane
+  static constexpr int DB = DP / 32;         // 32-wide blocks along D
+  static constexpr int CPR = D / VEC;        // 16-byte chunks per row
+
+  // XOR mask (in chunks) for a row; depends on row & 15 only
+  SA_DEV static int swz(int row) {
+    if constexpr (!SWZ) return 0;
+    else if constexpr (CPR >= 16) return ((row & 3) << 2) | ((row >> 2) & 3);
+    else return ((row >> 2) & 1) | (((row >> 3) & 1) << 1) | (((row >> 1) & 1) << 2);   // CPR == 8
+  }
+  // element offset of (row, element col) inside a tile
+  SA_DEV static int off(int row, int col) {
+    if constexpr (!SWZ) return row * PITCH + col;
+    else return row * PITCH + ((((col / VEC) ^ swz(row)) * VEC) | (col % VEC));
+  }
 };
 
 SA_DEV void mma(f32x16& acc, bf16x8 a, bf16x8 b) {
@@ -94,6 +121,11 @@ SA_DEV float half_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Block until every outstanding global load of this wave has returned (vmcnt = 0, the other
+// counters untouched).  Placed before a main loop so that the waits the compiler must insert
+// for loop-invariant operands do not also drain the prefetch loads issued inside the loop.
+SA_DEV void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 SA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 template <typename T> SA_DEV typename Elem<T>::Frag negate(typename Elem<T>::Frag f) {
@@ -112,34 +144,91 @@ SA_DEV typename Elem<T>::Frag lds_row_frag(const T* tile, int row, int g, int h)
   return *reinterpret_cast<const Frag*>(tile + row * PITCH + (g * 2 + h) * Elem<T>::VEC);
 }
 
+// The compiler's scheduler, left alone, issues each LDS read right before the MFMA that
+// consumes it and so exposes the full LDS latency once per MFMA.  pipeline() forces the
+// shape "fetch group n+1, then multiply group n" with scheduling fences between groups:
+// N items in groups of G, load(i) returns the fragment of item i, use(i, frag) consumes it.
+SA_DEV void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
+
+template <int N, int G, typename LoadF, typename UseF>
+SA_DEV void pipeline(LoadF&& load, UseF&& use) {
+  static_assert(N % G == 0, "items must fill whole groups");
+  using F = decltype(load(0));
+  constexpr int NG = N / G;
+  F buf[2][G];
+#pragma unroll
+  for (int j = 0; j < G; ++j) buf[0][j] = load(j);
+#pragma unroll
+  for (int grp = 0; grp < NG; ++grp) {
+    sched_fence();
+    if (grp + 1 < NG) {
+#pragma unroll
+      for (int j = 0; j < G; ++j) buf[(grp + 1) & 1][j] = load((grp + 1) * G + j);
+    }
+#pragma unroll
+    for (int j = 0; j < G; ++j) use(grp * G + j, buf[grp & 1][j]);
+  }
+  sched_fence();
+}
+
+// acc[nb] += A_nb * B for NB row blocks of a row-major LDS tile that share the register
+// fragments bf:  acc[nb][row r][col c] += sum_k tile[row0 + nb*32 + r][k] * B[k][c].
+template <typename T, int D, int NB, int NF>
+SA_DEV void mma_rows(f32x16 (&acc)[NB], const T* tile, int row0, const typename Elem<T>::Frag (&bf)[NF],
+                     int lane) {
+  using G_ = TileGeom<T, D>;
+  static_assert(NF == G_::NF, "one register fragment per 2*VEC slice of the head dimension");
+  constexpr int PITCH = G_::PITCH, VEC = Elem<T>::VEC;
+  const int c = lane & 31, h = lane >> 5;
+  constexpr int N = NB * NF, G = N < 4 ? N : 4;
+  // row0 is a multiple of 32, so the swizzle of this lane's rows depends on c alone
+  const T* base = tile + (row0 + c) * PITCH;
+  const int sw = G_::swz(c);
+  pipeline<N, G>(
+      [&](int it) {
+        const int nb = it / NF, g = it % NF;
+        return *reinterpret_cast<const typename Elem<T>::Frag*>(base + nb * 32 * PITCH + (((g * 2 + h) ^ sw) * VEC));
+      },
+      [&](int it, const typename Elem<T>::Frag& a) { mma(acc[it / NF], a, bf[it % NF]); });
+}
+
 // acc[m] += X^T * P for one 32-row block `rb` of a row-major LDS tile X[rows][cols]:
 //   acc[m][row x][col c] += sum_r X[rb*32 + r][m*32 + x] * P[r][c]
 // where P is a C fragment (its rows are the contraction index).  P is rounded to T
 // before the product, as the operand of a 16-bit MFMA must be.
-template <typename T, int PITCH, int NM>
+template <typename T, int D, int NM>
 SA_DEV void mma_tr(f32x16 (&acc)[NM], const T* X, int rb, const f32x16& P, int lane) {
   using E = Elem<T>;
+  using G_ = TileGeom<T, D>;
+  static_assert(NM == G_::DB, "one accumulator per 32-wide block of the head dimension");
+  constexpr int PITCH = G_::PITCH;
   if constexpr (E::HALF) {
+    using Frag = typename E::Frag;
     const int g16 = lane >> 4, j = lane & 15;
     const int h = g16 >> 1, mb = (g16 & 1) * 16;
-    // this lane's source address for the transposing read: row (j/4) of a 4-row run,
-    // 4 columns starting at 4*(j%4); the instruction hands lane j column j of the
-    // 4x16 block, i.e. 4 consecutive rows of one column.
-    const T* base = X + (rb * 32 + 4 * h + (j >> 2)) * PITCH + mb + 4 * (j & 3);
+    // This lane's source address for the transposing read: row (j/4) of a 4-row run, the
+    // 4 columns starting at 4*(j%4); the instruction hands lane j column j of the 4x16
+    // block, i.e. 4 consecutive rows of one column.  Two runs, 8 rows apart, make the
+    // 8 contraction slots of one fragment.
+    const int r_lo = 4 * h + (j >> 2);            // row inside a 16-row half, first run
+    const int col = mb + 4 * (j & 3);             // element column inside a 32-wide block
+    const T* blk = X + rb * 32 * PITCH;
+    Frag b[2];
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      typename E::Frag b;
+    for (int half = 0; half < 2; ++half)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) b[e] = (T)P[half * 8 + e];
-#pragma unroll
-      for (int m = 0; m < NM; ++m) {
-        const T* p0 = base + (half * 16) * PITCH + m * 32;
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p0));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p0 + 8 * PITCH));
-        s16x8 a8 = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        mma(acc[m], __builtin_bit_cast(typename E::Frag, a8), b);
-      }
-    }
+      for (int e = 0; e < 8; ++e) b[half][e] = (T)P[half * 8 + e];
+    constexpr int N = 2 * NM, G = N < 4 ? N : 4;
+    pipeline<N, G>(
+        [&](int it) {
+          const int half = it / NM, m = it % NM;
+          const T* p0 = blk + G_::off(half * 16 + r_lo, m * 32 + col);
+          const T* p1 = blk + G_::off(half * 16 + 8 + r_lo, m * 32 + col);
+          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p0));
+          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p1));
+          return __builtin_bit_cast(Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        },
+        [&](int it, const Frag& a) { mma(acc[it % NM], a, b[it / NM]); });
   } else {
     const int c = lane & 31, h = lane >> 5;
 #pragma unroll
@@ -182,7 +271,7 @@ template <typename T, int D, int ROWS, int NT> struct Stager {
       const int ch = tid + it * NT;
       if (TOTAL % NT == 0 || ch < TOTAL) {
         const int r = ch / CPR, col = (ch % CPR) * E::VEC;
-        *reinterpret_cast<Frag*>(tile + r * PITCH + col) = regs[it];
+        *reinterpret_cast<Frag*>(tile + TileGeom<T, D>::off(r, col)) = regs[it];
       }
     }
   }

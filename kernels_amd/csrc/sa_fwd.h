@@ -19,6 +19,7 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
   constexpr int TQ = NW * 32, NT = NW * 64, KBN = TK / 32;
   constexpr int PITCH = G::PITCH, NF = G::NF, DB = G::DB;
   constexpr int TILE = TK * PITCH;  // elements per staged K or V tile
+  constexpr float kRescaleGap = 8.0f;
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   T* smem = reinterpret_cast<T*>(smem_raw);  // [stage][K|V][TK][PITCH]
@@ -98,6 +99,7 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
   sv.load(vbase, p.v_st, kt0 * TK, T_ - 1, tid);
   sk.store(smem, tid);
   sv.store(smem + TILE, tid);
+  wait_all_loads();
   __syncthreads();
 
   for (int t = kt0; t < kt1; ++t) {
@@ -114,59 +116,74 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
     // S^T[key][q] = K Q^T
     f32x16 s[KBN];
 #pragma unroll
-    for (int kb = 0; kb < KBN; ++kb) {
+    for (int kb = 0; kb < KBN; ++kb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[kb][i] = 0.0f;
-#pragma unroll
-      for (int g = 0; g < NF; ++g) mma(s[kb], lds_row_frag<T, PITCH>(Kt, kb * 32 + c, g, h), qf[g]);
-    }
+    mma_rows<T, D>(s, Kt, 0, qf, lane);
 
+    // Online softmax in base 2 on the raw scores: p = exp2(s*sl2e - m).  The two halves of
+    // the wave hold disjoint keys of the same query, so only the max crosses lanes inside
+    // the loop.  The reference point m moves only when the tile's max exceeds it by more
+    // than kRescaleGap (p then stays below 2^kRescaleGap, harmless in fp32 and in the 16-bit
+    // operand of the next product); most tiles therefore skip the rescale of O entirely.
+    const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
+    float mx = -INFINITY;
+    if (interior) {
+#pragma unroll
+      for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = k0 + kb * 32 + crow(i, h);
+          mx = (key >= lo && key < hi) ? fmaxf(mx, s[kb][i]) : mx;
+        }
+    }
+    mx = half_max(mx) * sl2e;                 // -inf when no key of this tile is visible
+    const bool move = mx > m_run + kRescaleGap;   // false for mx = -inf or NaN
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      const float m_new = move ? mx : m_run;
+      // m_run = -inf gives alpha = 0 (the accumulators are 0 then); lanes that stay put get 1
+      const float alpha = move ? fast_exp2(m_run - mx) : 1.0f;
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int m = 0; m < DB; ++m)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[m][i] *= alpha;
+    }
+    // a query that has seen no key yet keeps m_run = -inf; use 0 there so that exp2 gets a
+    // finite argument (its keys in this tile are all masked, so p is forced to 0 below)
+    const float m_use = m_run == -INFINITY ? 0.0f : m_run;
+    float rs = 0.0f;
 #pragma unroll
     for (int kb = 0; kb < KBN; ++kb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[kb][i] *= sl2e;
-
-    const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
+      for (int i = 0; i < 16; ++i) {
+        const float e = fast_exp2(__builtin_fmaf(s[kb][i], sl2e, -m_use));
+        s[kb][i] = e;
+      }
     if (!interior) {
 #pragma unroll
       for (int kb = 0; kb < KBN; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int key = k0 + kb * 32 + crow(i, h);
-          if (key < lo || key >= hi) s[kb][i] = -INFINITY;
+          s[kb][i] = (key >= lo && key < hi) ? s[kb][i] : 0.0f;
         }
     }
-
-    // online softmax in base 2; the two halves of the wave hold disjoint keys of
-    // the same query, so only the max has to cross lanes inside the loop
-    float mx = -INFINITY;
 #pragma unroll
     for (int kb = 0; kb < KBN; ++kb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
-    mx = half_max(mx);
-    const float m_new = fmaxf(m_run, mx);
-    const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
-    const float alpha = fast_exp2(m_run - m_safe);
-    float rs = 0.0f;
-#pragma unroll
-    for (int kb = 0; kb < KBN; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float e = fast_exp2(s[kb][i] - m_safe);
-        s[kb][i] = e;
-        rs += e;
-      }
-    l_run = l_run * alpha + rs;
-    m_run = m_new;
-#pragma unroll
-    for (int m = 0; m < DB; ++m)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[m][i] *= alpha;
+      for (int i = 0; i < 16; ++i) rs += s[kb][i];
+    l_run += rs;
 
     // O^T[d][q] += V^T P^T
 #pragma unroll
-    for (int kb = 0; kb < KBN; ++kb) mma_tr<T, PITCH, DB>(oacc, Vt, kb, s[kb], lane);
+    for (int kb = 0; kb < KBN; ++kb) mma_tr<T, D>(oacc, Vt, kb, s[kb], lane);
 
     if (more) {
       T* nxt = smem + (cur ^ 1) * 2 * TILE;

@@ -1,6 +1,7 @@
 // Kernel instantiations for one element type and one kernel family.
 // Compiled once per (SA_DTYPE_ID, SA_KIND) pair so that the families build in parallel.
 //   SA_DTYPE_ID: 0 fp32, 1 fp16, 2 bf16        SA_KIND: 0 forward, 1 delta + dQ, 2 dK/dV
+//   SA_DGROUP: 0 head dims 16..128, 1 head dim 256
 #include <mutex>
 #include "sa_launch.h"
 #if SA_KIND == 0
@@ -33,15 +34,24 @@ template <typename K> static int prepare(K kernel, size_t lds_bytes, std::once_f
 
 static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// SA_DGROUP 0 holds head dimensions 16..128, SA_DGROUP 1 holds 256 (built with different
+// compiler options, see the Makefile).
+#if SA_DGROUP == 0
 #define SA_FOR_EACH_D(X) \
   switch (D) {           \
     case 16: X(16);      \
     case 32: X(32);      \
     case 64: X(64);      \
     case 128: X(128);    \
+    default: return SA_ERR_HEAD_DIM; \
+  }
+#else
+#define SA_FOR_EACH_D(X) \
+  switch (D) {           \
     case 256: X(256);    \
     default: return SA_ERR_HEAD_DIM; \
   }
+#endif
 
 #if SA_KIND == 0
 template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
@@ -57,7 +67,7 @@ template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
   return (int)hipGetLastError();
 }
-template <> int launch_fwd<ElemT>(const FwdParams& p, int D, hipStream_t st) {
+template <> int launch_fwd<ElemT, SA_DGROUP>(const FwdParams& p, int D, hipStream_t st) {
 #define X(d) return fwd_d<d>(p, st)
   SA_FOR_EACH_D(X)
 #undef X
@@ -71,7 +81,7 @@ template <int D> static int delta_d(const DeltaParams& p, hipStream_t st) {
   hipLaunchKernelGGL((delta_kernel<ElemT, D>), dim3((unsigned)blocks), dim3(256), 0, st, p);
   return (int)hipGetLastError();
 }
-template <> int launch_delta<ElemT>(const DeltaParams& p, int D, hipStream_t st) {
+template <> int launch_delta<ElemT, SA_DGROUP>(const DeltaParams& p, int D, hipStream_t st) {
 #define X(d) return delta_d<d>(p, st)
   SA_FOR_EACH_D(X)
 #undef X
@@ -89,7 +99,7 @@ template <int D> static int dq_d(BwdParams p, hipStream_t st) {
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
   return (int)hipGetLastError();
 }
-template <> int launch_dq<ElemT>(const BwdParams& p, int D, hipStream_t st) {
+template <> int launch_dq<ElemT, SA_DGROUP>(const BwdParams& p, int D, hipStream_t st) {
 #define X(d) return dq_d<d>(p, st)
   SA_FOR_EACH_D(X)
 #undef X
@@ -109,7 +119,7 @@ template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
   return (int)hipGetLastError();
 }
-template <> int launch_dkdv<ElemT>(const BwdParams& p, int D, hipStream_t st) {
+template <> int launch_dkdv<ElemT, SA_DGROUP>(const BwdParams& p, int D, hipStream_t st) {
 #define X(d) return dkdv_d<d>(p, st)
   SA_FOR_EACH_D(X)
 #undef X

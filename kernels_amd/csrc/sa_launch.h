@@ -9,10 +9,10 @@
 namespace sa {
 
 
-template <typename T> int launch_fwd(const FwdParams& p, int D, hipStream_t st);
-template <typename T> int launch_delta(const DeltaParams& p, int D, hipStream_t st);
-template <typename T> int launch_dq(const BwdParams& p, int D, hipStream_t st);
-template <typename T> int launch_dkdv(const BwdParams& p, int D, hipStream_t st);
+template <typename T, int DGROUP> int launch_fwd(const FwdParams& p, int D, hipStream_t st);
+template <typename T, int DGROUP> int launch_delta(const DeltaParams& p, int D, hipStream_t st);
+template <typename T, int DGROUP> int launch_dq(const BwdParams& p, int D, hipStream_t st);
+template <typename T, int DGROUP> int launch_dkdv(const BwdParams& p, int D, hipStream_t st);
 
 // tile sizes, shared between the launchers and sa_query()
 template <typename T> struct Cfg {
