@@ -373,4 +373,309 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Variants for 16-bit elements with swizzled tiles (D = 64 or 128): tiles arrive by
+// asynchronous global->LDS copies into a ring of NST stages, one barrier per tile.
+// ---------------------------------------------------------------------------------------
+
+template <typename T, int D, int NW, int TK, int NST>
+__global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
+  using E = Elem<T>;
+  using G = TileGeom<T, D>;
+  using Frag = typename E::Frag;
+  static_assert(G::SWZ && (NST == 2 || NST == 3), "swizzled 16-bit tiles, 2 or 3 stages");
+  constexpr int TQ = NW * 32, NT = NW * 64, KBN = TK / 32;
+  constexpr int NF = G::NF, DB = G::DB;
+  constexpr int TILE = TK * D, STAGE = 2 * TILE;
+  using Loader = AsyncTile<T, D, TK, NW>;
+  constexpr int LPT = 2 * Loader::PER_WAVE;
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  T* smem = reinterpret_cast<T*>(smem_raw);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int bid = xcd_remap(blockIdx.x, gridDim.x);
+  const int qt = bid % p.n_tiles;
+  const int bh = bid / p.n_tiles;
+  const int hd = bh % p.H, b = bh / p.H;
+  const int T_ = p.T, C = p.C, R = p.R;
+
+  int L = T_;
+  if (p.lens) {
+    L = p.lens[(int64_t)b * p.lens_stride];
+    L = L < 0 ? 0 : (L > T_ ? T_ : L);
+  }
+  const int q0 = qt * TQ;
+  T* dq_base = reinterpret_cast<T*>(p.dq) + (int64_t)bh * T_ * D;
+  const int q_end = q0 + TQ < T_ ? q0 + TQ : T_;
+  if (q0 >= L) {
+    zero_rows<T, D, NT>(dq_base, q0, q_end, tid);
+    return;
+  }
+
+  const int qrow = q0 + wave * 32 + c;
+  const int qe = qrow < L ? qrow : L - 1;
+  const int qchunk = qe / C;
+  const int lo = (qchunk > R ? qchunk - R : 0) * C;
+  const int hi = (qchunk + 1) * C < L ? (qchunk + 1) * C : L;
+  const int wq_first = q0 + wave * 32 < L ? q0 + wave * 32 : L - 1;
+  const int wq_last = q0 + wave * 32 + 31 < L ? q0 + wave * 32 + 31 : L - 1;
+  const int hi_min = (wq_first / C + 1) * C < L ? (wq_first / C + 1) * C : L;
+  const int lo_max = (wq_last / C > R ? wq_last / C - R : 0) * C;
+  const int gq_last = q0 + TQ - 1 < L ? q0 + TQ - 1 : L - 1;
+  const int lo_wg = (q0 / C > R ? q0 / C - R : 0) * C;
+  const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
+  const int kt0 = lo_wg / TK, kt1 = (hi_wg + TK - 1) / TK;
+
+  const float sl2e = fabsf(p.scale_log2e);
+  const bool neg = p.scale_log2e < 0.0f;
+
+  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh;
+  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh;
+  auto issue_tile = [&](int t) {
+    T* st = smem + ((t - kt0) % NST) * STAGE;
+    Loader::issue(kbase, p.k_st, t * TK, T_ - 1, st, wave, lane);
+    Loader::issue(vbase, p.v_st, t * TK, T_ - 1, st + TILE, wave, lane);
+  };
+#pragma unroll
+  for (int i = 0; i < NST - 1; ++i)
+    if (kt0 + i < kt1) issue_tile(kt0 + i);
+
+  Frag qf[NF], gf[NF];
+  float lse_q, delta_q;
+  {
+    const int qr = qrow < T_ ? qrow : T_ - 1;
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh +
+                  (int64_t)qr * p.q_st;
+    const T* gp = reinterpret_cast<const T*>(p.d_o) + (int64_t)b * p.do_sb + (int64_t)hd * p.do_sh +
+                  (int64_t)qr * p.do_st;
+#pragma unroll
+    for (int g = 0; g < NF; ++g) {
+      qf[g] = *reinterpret_cast<const Frag*>(qp + (g * 2 + h) * E::VEC);
+      if (neg) qf[g] = negate<T>(qf[g]);
+      gf[g] = *reinterpret_cast<const Frag*>(gp + (g * 2 + h) * E::VEC);
+    }
+    lse_q = qrow < L ? p.lse[(int64_t)bh * T_ + qr] : INFINITY;   // rows past L: P = exp2(-inf) = 0
+    delta_q = p.delta[(int64_t)bh * T_ + qr];
+  }
+
+  f32x16 acc[DB];
+#pragma unroll
+  for (int m = 0; m < DB; ++m)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
+  wait_all_loads();
+
+  for (int t = kt0; t < kt1; ++t) {
+    if (NST == 3 && t + 1 < kt1) wait_loads<LPT>();
+    else wait_loads<0>();
+    __syncthreads();
+    if (t + NST - 1 < kt1) issue_tile(t + NST - 1);
+
+    const T* Kt = smem + ((t - kt0) % NST) * STAGE;
+    const T* Vt = Kt + TILE;
+    const int k0 = t * TK;
+    const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
+
+#pragma unroll
+    for (int kb = 0; kb < KBN; ++kb) {
+      f32x16 s[1], dp[1];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[0][i] = 0.0f, dp[0][i] = 0.0f;
+      mma_rows<T, D>(s, Kt, kb * 32, qf, lane);
+      mma_rows<T, D>(dp, Vt, kb * 32, gf, lane);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float pr = fast_exp2(__builtin_fmaf(s[0][i], sl2e, -lse_q));
+        s[0][i] = pr * (dp[0][i] - delta_q);
+      }
+      if (!interior) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = k0 + kb * 32 + crow(i, h);
+          s[0][i] = (key < lo || key >= hi) ? 0.0f : s[0][i];
+        }
+      }
+      mma_tr<T, D>(acc, Kt, kb, s[0], lane);   // dQ^T[d][q] += K^T dS^T
+    }
+  }
+
+  if (qrow < T_) {
+    if (qrow >= L) {
+#pragma unroll
+      for (int m = 0; m < DB; ++m)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
+    }
+    store_acc_T<T, D, DB>(dq_base + (int64_t)qrow * D, acc, p.scale, h);
+  }
+}
+
+template <typename T, int D, int NW, int TQ, int NST>
+__global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
+  using E = Elem<T>;
+  using G = TileGeom<T, D>;
+  using Frag = typename E::Frag;
+  static_assert(G::SWZ && (NST == 2 || NST == 3), "swizzled 16-bit tiles, 2 or 3 stages");
+  constexpr int TKB = NW * 32, NT = NW * 64, QBN = TQ / 32;
+  constexpr int NF = G::NF, DB = G::DB;
+  constexpr int TILE = TQ * D;
+  constexpr int RPW = TQ / NW;   // rows of lse / delta each wave stages
+  static_assert(TQ % NW == 0 && RPW % 4 == 0 && 2 * RPW <= 64, "lse/delta staging: one instruction per wave");
+  // stage layout: [Q tile][dO tile][NW chunks of {lse[RPW], delta[RPW]}]
+  constexpr int STAGE_BYTES = 2 * TILE * (int)sizeof(T) + 2 * TQ * (int)sizeof(float);
+  using Loader = AsyncTile<T, D, TQ, NW>;
+  constexpr int LPT = 2 * Loader::PER_WAVE + 1;
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int bid = xcd_remap(blockIdx.x, gridDim.x);
+  const int kt = bid % p.n_tiles;
+  const int bh = bid / p.n_tiles;
+  const int hd = bh % p.H, b = bh / p.H;
+  const int T_ = p.T, C = p.C, R = p.R;
+
+  int L = T_;
+  if (p.lens) {
+    L = p.lens[(int64_t)b * p.lens_stride];
+    L = L < 0 ? 0 : (L > T_ ? T_ : L);
+  }
+  const int k0 = kt * TKB;
+  T* dk_base = reinterpret_cast<T*>(p.dk) + (int64_t)bh * T_ * D;
+  T* dv_base = reinterpret_cast<T*>(p.dv) + (int64_t)bh * T_ * D;
+  const int k_end = k0 + TKB < T_ ? k0 + TKB : T_;
+  if (k0 >= L) {
+    zero_rows<T, D, NT>(dk_base, k0, k_end, tid);
+    zero_rows<T, D, NT>(dv_base, k0, k_end, tid);
+    return;
+  }
+
+  auto win_lo = [&](int key) { return (key / C) * C; };
+  auto win_hi = [&](int key) {
+    const int64_t e = ((int64_t)(key / C) + R + 1) * (int64_t)C;
+    return e < (int64_t)L ? (int)e : L;
+  };
+  const int krow = k0 + wave * 32 + c;
+  const int ke = krow < L ? krow : L - 1;
+  const int qlo = win_lo(ke), qhi = win_hi(ke);
+  const int wk_first = k0 + wave * 32 < L ? k0 + wave * 32 : L - 1;
+  const int wk_last = k0 + wave * 32 + 31 < L ? k0 + wave * 32 + 31 : L - 1;
+  const int qhi_min = win_hi(wk_first), qlo_max = win_lo(wk_last);
+  const int gk_last = k0 + TKB - 1 < L ? k0 + TKB - 1 : L - 1;
+  const int qt0 = win_lo(k0) / TQ, qt1 = (win_hi(gk_last) + TQ - 1) / TQ;
+
+  const float sl2e = fabsf(p.scale_log2e);
+  const bool neg = p.scale_log2e < 0.0f;
+
+  const T* qbase = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh;
+  const T* gbase = reinterpret_cast<const T*>(p.d_o) + (int64_t)b * p.do_sb + (int64_t)hd * p.do_sh;
+  const float* lse_base = p.lse + (int64_t)bh * T_;
+  const float* delta_base = p.delta + (int64_t)bh * T_;
+  auto stage_ptr = [&](int t) { return smem_raw + ((t - qt0) % NST) * STAGE_BYTES; };
+  auto issue_tile = [&](int t) {
+    T* st = reinterpret_cast<T*>(stage_ptr(t));
+    Loader::issue(qbase, p.q_st, t * TQ, T_ - 1, st, wave, lane);
+    Loader::issue(gbase, p.do_st, t * TQ, T_ - 1, st + TILE, wave, lane);
+    // lanes [0, RPW) fetch lse, lanes [RPW, 2*RPW) fetch delta of this wave's RPW rows
+    if (lane < 2 * RPW) {
+      int r = t * TQ + wave * RPW + (lane % RPW);
+      r = r < T_ ? r : T_ - 1;
+      const float* src = (lane < RPW ? lse_base : delta_base) + r;
+      float* dst = reinterpret_cast<float*>(stage_ptr(t) + 2 * TILE * sizeof(T)) + wave * 2 * RPW;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (SA_LDS void*)dst, 4, 0, 0);
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < NST - 1; ++i)
+    if (qt0 + i < qt1) issue_tile(qt0 + i);
+
+  Frag kf[NF], vf[NF];
+  {
+    const int kr = krow < T_ ? krow : T_ - 1;
+    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh +
+                  (int64_t)kr * p.k_st;
+    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh +
+                  (int64_t)kr * p.v_st;
+#pragma unroll
+    for (int g = 0; g < NF; ++g) {
+      kf[g] = *reinterpret_cast<const Frag*>(kp + (g * 2 + h) * E::VEC);
+      if (neg) kf[g] = negate<T>(kf[g]);
+      vf[g] = *reinterpret_cast<const Frag*>(vp + (g * 2 + h) * E::VEC);
+    }
+  }
+
+  f32x16 dk[DB], dv[DB];
+#pragma unroll
+  for (int m = 0; m < DB; ++m)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
+  wait_all_loads();
+
+  for (int t = qt0; t < qt1; ++t) {
+    if (NST == 3 && t + 1 < qt1) wait_loads<LPT>();
+    else wait_loads<0>();
+    __syncthreads();
+    if (t + NST - 1 < qt1) issue_tile(t + NST - 1);
+
+    const T* Qt = reinterpret_cast<const T*>(stage_ptr(t));
+    const T* Gt = Qt + TILE;
+    const float* ld_t = reinterpret_cast<const float*>(stage_ptr(t) + 2 * TILE * sizeof(T));
+    const int qs = t * TQ;
+    const bool interior = (qs >= qlo_max) && (qs + TQ <= qhi_min);
+
+#pragma unroll
+    for (int qb = 0; qb < QBN; ++qb) {
+      f32x16 s[1], dp[1];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[0][i] = 0.0f, dp[0][i] = 0.0f;
+      mma_rows<T, D>(s, Qt, qb * 32, kf, lane);    // S[q][key] = Q K^T
+      mma_rows<T, D>(dp, Gt, qb * 32, vf, lane);   // dP[q][key] = dO V^T
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int r = qb * 32 + 8 * g4 + 4 * h;     // tile row of 4 consecutive C-fragment rows
+        const float* chunk = ld_t + (r / RPW) * 2 * RPW + (r % RPW);
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(chunk);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(chunk + RPW);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = 4 * g4 + e;
+          const float pr = fast_exp2(__builtin_fmaf(s[0][i], sl2e, -l4[e]));
+          s[0][i] = pr;
+          dp[0][i] = pr * (dp[0][i] - d4[e]);
+        }
+      }
+      if (!interior) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int qr = qs + qb * 32 + crow(i, h);
+          const bool ok = qr >= qlo && qr < qhi;
+          s[0][i] = ok ? s[0][i] : 0.0f;
+          dp[0][i] = ok ? dp[0][i] : 0.0f;
+        }
+      }
+      mma_tr<T, D>(dv, Gt, qb, s[0], lane);    // dV^T[d][key] += dO^T P
+      mma_tr<T, D>(dk, Qt, qb, dp[0], lane);   // dK^T[d][key] += Q^T dS
+    }
+  }
+
+  if (krow < T_) {
+    if (krow >= L) {
+#pragma unroll
+      for (int m = 0; m < DB; ++m)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
+    }
+    store_acc_T<T, D, DB>(dk_base + (int64_t)krow * D, dk, p.scale, h);
+    store_acc_T<T, D, DB>(dv_base + (int64_t)krow * D, dv, 1.0f, h);
+  }
+}
+
 }  // namespace sa

@@ -128,6 +128,10 @@ SA_DEV void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
 SA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// max(a, b) as median(a, b, +inf): one v_med3_f32, with none of the input canonicalisation
+// that fmaxf() costs per operand.
+SA_DEV float fast_max(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, INFINITY); }
+
 template <typename T> SA_DEV typename Elem<T>::Frag negate(typename Elem<T>::Frag f) {
   u32x4 u = __builtin_bit_cast(u32x4, f);
   u ^= Elem<T>::SIGN;
@@ -239,6 +243,123 @@ SA_DEV void mma_tr(f32x16 (&acc)[NM], const T* X, int rb, const f32x16& P, int l
         acc[m] = __builtin_amdgcn_mfma_f32_32x32x2f32(row[m * 32], P[i], acc[m], 0, 0, 0);
     }
   }
+}
+
+// Variants of the two products for a wave that owns NQ 32-wide blocks of the "owner" index:
+// every fragment fetched from LDS is multiplied against NQ register fragments, which
+// divides the LDS traffic per MFMA by NQ.
+template <typename T, int D, int NQ, int NB, int NF>
+SA_DEV void mma_rows_n(f32x16 (&acc)[NQ][NB], const T* tile, int row0,
+                       const typename Elem<T>::Frag (&bf)[NQ][NF], int lane) {
+  using G_ = TileGeom<T, D>;
+  static_assert(NF == G_::NF, "one register fragment per 2*VEC slice of the head dimension");
+  constexpr int PITCH = G_::PITCH, VEC = Elem<T>::VEC;
+  const int c = lane & 31, h = lane >> 5;
+  constexpr int N = NB * NF, G = N < 4 ? N : 4;
+  const T* base = tile + (row0 + c) * PITCH;
+  const int sw = G_::swz(c);
+  pipeline<N, G>(
+      [&](int it) {
+        const int nb = it / NF, g = it % NF;
+        return *reinterpret_cast<const typename Elem<T>::Frag*>(base + nb * 32 * PITCH + (((g * 2 + h) ^ sw) * VEC));
+      },
+      [&](int it, const typename Elem<T>::Frag& a) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) mma(acc[q][it / NF], a, bf[q][it % NF]);
+      });
+}
+
+// Round a C fragment to T and pack it as the two B fragments (16 contraction rows each)
+// that mma_tr_n consumes.
+template <typename T> SA_DEV void pack_c(typename Elem<T>::Frag (&b)[2], const f32x16& P) {
+#pragma unroll
+  for (int half = 0; half < 2; ++half)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[half][e] = (T)P[half * 8 + e];
+}
+
+// 16-bit only: acc[q][m] += X^T * B[q] for 32-row block rb of tile X, B[q] packed by pack_c.
+template <typename T, int D, int NQ, int NM>
+SA_DEV void mma_tr_n(f32x16 (&acc)[NQ][NM], const T* X, int rb, const typename Elem<T>::Frag (&b)[NQ][2],
+                     int lane) {
+  using E = Elem<T>;
+  using G_ = TileGeom<T, D>;
+  using Frag = typename E::Frag;
+  static_assert(E::HALF && NM == G_::DB, "transposing reads exist for 16-bit elements only");
+  constexpr int PITCH = G_::PITCH;
+  const int g16 = lane >> 4, j = lane & 15;
+  const int h = g16 >> 1, mb = (g16 & 1) * 16;
+  const int r_lo = 4 * h + (j >> 2);
+  const int col = mb + 4 * (j & 3);
+  const T* blk = X + rb * 32 * PITCH;
+  constexpr int N = 2 * NM, G = N < 4 ? N : 4;
+  pipeline<N, G>(
+      [&](int it) {
+        const int half = it / NM, m = it % NM;
+        const T* p0 = blk + G_::off(half * 16 + r_lo, m * 32 + col);
+        const T* p1 = blk + G_::off(half * 16 + 8 + r_lo, m * 32 + col);
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p0));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p1));
+        return __builtin_bit_cast(Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      },
+      [&](int it, const Frag& a) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) mma(acc[q][it % NM], a, b[q][it / NM]);
+      });
+}
+
+// Asynchronous copy of a [ROWS][D] row-major global tile into a swizzled LDS tile with
+// global_load_lds_dwordx4: the data never passes through registers.  One instruction moves
+// 1 KiB (64 lanes x 16 bytes) to consecutive LDS addresses, i.e. 1024/(2*D) whole rows; lane l
+// therefore fetches, for physical chunk l % CPR of its row, the logical chunk that the swizzle
+// maps there.  The NW waves of a workgroup interleave instruction by instruction.  Completion
+// is tracked by vmcnt; visibility to the other waves needs a barrier after the wait.
+template <typename T, int D, int ROWS, int NW> struct AsyncTile {
+  using G_ = TileGeom<T, D>;
+  static_assert(G_::SWZ, "asynchronous tiles use the swizzled layout");
+  static constexpr int ROW_BYTES = D * (int)sizeof(T);
+  static constexpr int RPI = 1024 / ROW_BYTES;             // rows per instruction
+  static constexpr int NI = ROWS / RPI;                     // instructions per tile
+  static_assert(ROWS % (RPI * NW) == 0, "tile must split evenly over the waves");
+  static constexpr int PER_WAVE = NI / NW;                  // instructions per wave per tile
+
+  // Issue this wave's share of the tile whose first row is row0 (rows clamped to last_row).
+  // The address of a lane is (wave-uniform 64-bit row base) + (32-bit lane offset): the
+  // uniform part is scalar arithmetic, and the lane offset does not change from tile to tile
+  // unless the tile hangs over the end of the sequence.
+  SA_DEV static void issue(const T* gbase, int64_t row_stride, int row0, int last_row, T* tile, int wave,
+                           int lane) {
+    const int lrow = lane / G_::CPR, pch = lane % G_::CPR;
+    const uint32_t rs = (uint32_t)row_stride;
+    if (row0 + ROWS - 1 <= last_row) {
+#pragma unroll
+      for (int i = 0; i < PER_WAVE; ++i) {
+        const int rb = (i * NW + wave) * RPI;                // wave-uniform first row of this instruction
+        const uint32_t loff = (uint32_t)lrow * rs + (uint32_t)((pch ^ G_::swz(rb + lrow)) * Elem<T>::VEC);
+        const T* src = gbase + (int64_t)(row0 + rb) * row_stride + loff;
+        T* dst = tile + rb * D;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (SA_LDS void*)dst, 16, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PER_WAVE; ++i) {
+        const int rb = (i * NW + wave) * RPI;
+        int gr = row0 + rb + lrow;
+        gr = gr < last_row ? gr : last_row;
+        const T* src = gbase + (int64_t)gr * row_stride + ((pch ^ G_::swz(rb + lrow)) * Elem<T>::VEC);
+        T* dst = tile + rb * D;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (SA_LDS void*)dst, 16, 0, 0);
+      }
+    }
+  }
+};
+
+// s_waitcnt vmcnt(N), other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
+template <int N> SA_DEV void wait_loads() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
 // Cooperative copy of a [ROWS][D] row-major global tile into registers and on into an

@@ -102,6 +102,12 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
   wait_all_loads();
   __syncthreads();
 
+#ifdef SA_DBG_TIMING
+  long long tacc[6] = {0,0,0,0,0,0}; long long tp = __builtin_readcyclecounter();
+#define TICK(i) { long long tn = __builtin_readcyclecounter(); tacc[i] += tn - tp; tp = tn; }
+#else
+#define TICK(i)
+#endif
   for (int t = kt0; t < kt1; ++t) {
     const int cur = (t - kt0) & 1;
     const T* Kt = smem + cur * 2 * TILE;
@@ -112,6 +118,7 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
       sv.load(vbase, p.v_st, (t + 1) * TK, T_ - 1, tid);
     }
     const int k0 = t * TK;
+    TICK(0)
 
     // S^T[key][q] = K Q^T
     f32x16 s[KBN];
@@ -121,6 +128,7 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
       for (int i = 0; i < 16; ++i) s[kb][i] = 0.0f;
     mma_rows<T, D>(s, Kt, 0, qf, lane);
 
+    TICK(1)
     // Online softmax in base 2 on the raw scores: p = exp2(s*sl2e - m).  The two halves of
     // the wave hold disjoint keys of the same query, so only the max crosses lanes inside
     // the loop.  The reference point m moves only when the tile's max exceeds it by more
@@ -181,19 +189,31 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
       for (int i = 0; i < 16; ++i) rs += s[kb][i];
     l_run += rs;
 
+    TICK(2)
     // O^T[d][q] += V^T P^T
 #pragma unroll
     for (int kb = 0; kb < KBN; ++kb) mma_tr<T, D>(oacc, Vt, kb, s[kb], lane);
 
+    TICK(3)
     if (more) {
       T* nxt = smem + (cur ^ 1) * 2 * TILE;
       sk.store(nxt, tid);
       sv.store(nxt + TILE, tid);
     }
+    TICK(4)
     __syncthreads();
+    TICK(5)
   }
 
   // ---- epilogue --------------------------------------------------------------------
+#ifdef SA_DBG_TIMING
+  if (lse_base && lane < 6) {
+    long long tv = lane == 0 ? tacc[0] : lane == 1 ? tacc[1] : lane == 2 ? tacc[2] : lane == 3 ? tacc[3] : lane == 4 ? tacc[4] : tacc[5];
+    m_run = (float)tv / (float)(kt1 - kt0);
+    l_run = 0.5f;
+  }
+  if (lse_base && lane >= 32 && lane < 38) l_run = 0.5f;
+#endif
   const float l_tot = half_sum(l_run);
   const bool valid = qrow < L;
   if (qrow < T_) {
@@ -206,6 +226,253 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
     }
     store_acc_T<T, D, DB>(o_base + (int64_t)qrow * D, oacc, inv, h);
     if (lse_base && h == 0) lse_base[qrow] = valid ? m_run + __builtin_amdgcn_logf(l_tot) : 0.0f;
+  }
+}
+
+// Forward kernel for 16-bit elements with swizzled tiles (D = 64 or 128).
+//
+// Same algorithm as fwd_kernel, different resource balance: each wave owns QB blocks of 32
+// queries, so every K / V fragment fetched from LDS feeds QB MFMAs (the transposing V reads
+// are 8-byte LDS reads and would otherwise cap the second product well below the MFMA
+// rate); K and V tiles are brought in by asynchronous global->LDS copies into a ring of NST
+// stages, NST-1 tiles ahead of the compute, with one barrier per key tile.
+template <typename T, int D, int QB, int NW, int TK, int NST>
+__global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
+  using E = Elem<T>;
+  using G = TileGeom<T, D>;
+  using Frag = typename E::Frag;
+  static_assert(G::SWZ && (NST == 2 || NST == 3), "swizzled 16-bit tiles, 2 or 3 stages");
+  constexpr int WQ = QB * 32, TQ = NW * WQ, NT = NW * 64, KBN = TK / 32;
+  constexpr int NF = G::NF, DB = G::DB;
+  constexpr int TILE = TK * D;            // elements per K or V tile
+  constexpr int STAGE = 2 * TILE;
+  constexpr float kRescaleGap = 8.0f;
+  using Loader = AsyncTile<T, D, TK, NW>;
+  constexpr int LPT = 2 * Loader::PER_WAVE;   // async loads per wave per stage (K and V)
+
+  extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+  T* smem = reinterpret_cast<T*>(smem_raw);  // [stage][K|V][TK][D]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, c = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int bid = xcd_remap(blockIdx.x, gridDim.x);
+  const int qt = bid % p.n_tiles;
+  const int bh = bid / p.n_tiles;
+  const int hd = bh % p.H, b = bh / p.H;
+  const int T_ = p.T, C = p.C, R = p.R;
+
+  int L = T_;
+  if (p.lens) {
+    L = p.lens[(int64_t)b * p.lens_stride];
+    L = L < 0 ? 0 : (L > T_ ? T_ : L);
+  }
+  const int q0 = qt * TQ;
+  T* o_base = reinterpret_cast<T*>(p.o) + (int64_t)bh * T_ * D;
+  float* lse_base = p.lse ? p.lse + (int64_t)bh * T_ : nullptr;
+  const int q_end = q0 + TQ < T_ ? q0 + TQ : T_;
+  if (q0 >= L) {
+    zero_rows<T, D, NT>(o_base, q0, q_end, tid);
+    if (lse_base)
+      for (int r = q0 + tid; r < q_end; r += NT) lse_base[r] = 0.0f;
+    return;
+  }
+
+  // ---- per-lane queries (one per owned block) and their key windows -----------------
+  int qrow[QB], lo[QB], hi[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    qrow[qb] = q0 + wave * WQ + qb * 32 + c;
+    const int qe = qrow[qb] < L ? qrow[qb] : L - 1;
+    const int qchunk = qe / C;
+    lo[qb] = (qchunk > R ? qchunk - R : 0) * C;
+    hi[qb] = (qchunk + 1) * C < L ? (qchunk + 1) * C : L;
+  }
+  const int wq_first = q0 + wave * WQ < L ? q0 + wave * WQ : L - 1;
+  const int wq_last = q0 + wave * WQ + WQ - 1 < L ? q0 + wave * WQ + WQ - 1 : L - 1;
+  const int hi_min = (wq_first / C + 1) * C < L ? (wq_first / C + 1) * C : L;
+  const int lo_max = (wq_last / C > R ? wq_last / C - R : 0) * C;
+  const int gq_last = q0 + TQ - 1 < L ? q0 + TQ - 1 : L - 1;
+  const int lo_wg = (q0 / C > R ? q0 / C - R : 0) * C;
+  const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
+  const int kt0 = lo_wg / TK, kt1 = (hi_wg + TK - 1) / TK;
+
+  const float sl2e = fabsf(p.scale_log2e);
+  const bool neg = p.scale_log2e < 0.0f;
+
+  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh;
+  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh;
+  auto issue_tile = [&](int t) {
+    T* st = smem + ((t - kt0) % NST) * STAGE;
+    Loader::issue(kbase, p.k_st, t * TK, T_ - 1, st, wave, lane);
+    Loader::issue(vbase, p.v_st, t * TK, T_ - 1, st + TILE, wave, lane);
+  };
+  // prologue: NST-1 tiles in flight
+#pragma unroll
+  for (int i = 0; i < NST - 1; ++i)
+    if (kt0 + i < kt1) issue_tile(kt0 + i);
+
+  Frag qf[QB][NF];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    const int qr = qrow[qb] < T_ ? qrow[qb] : T_ - 1;
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh +
+                  (int64_t)qr * p.q_st;
+#pragma unroll
+    for (int g = 0; g < NF; ++g) {
+      qf[qb][g] = *reinterpret_cast<const Frag*>(qp + (g * 2 + h) * E::VEC);
+      if (neg) qf[qb][g] = negate<T>(qf[qb][g]);
+    }
+  }
+
+  f32x16 oacc[QB][DB];
+  float m_run[QB], l_run[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    m_run[qb] = -INFINITY;
+    l_run[qb] = 0.0f;
+#pragma unroll
+    for (int m = 0; m < DB; ++m)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[qb][m][i] = 0.0f;
+  }
+  wait_all_loads();   // Q fragments (and, as loads complete in order, the first tiles)
+
+#undef TICK
+#ifdef SA_DBG_TIMING
+  long long tacc[6] = {0,0,0,0,0,0}; long long tp = __builtin_readcyclecounter();
+#define TICK(i) { long long tn = __builtin_readcyclecounter(); tacc[i] += tn - tp; tp = tn; }
+#else
+#define TICK(i)
+#endif
+  for (int t = kt0; t < kt1; ++t) {
+    // tile t has landed once at most the younger tiles' loads are outstanding
+    if (NST == 3 && t + 1 < kt1) wait_loads<LPT>();
+    else wait_loads<0>();
+    TICK(0)
+    __syncthreads();   // every wave's share is visible; stage (t-1) % NST is free again
+    TICK(1)
+#ifndef SA_DBG_NOLOAD
+    if (t + NST - 1 < kt1) issue_tile(t + NST - 1);
+#endif
+
+    const T* Kt = smem + ((t - kt0) % NST) * STAGE;
+    const T* Vt = Kt + TILE;
+    const int k0 = t * TK;
+    TICK(5)
+
+    // S^T[key][q] = K Q^T for the QB query blocks
+    f32x16 s[QB][KBN];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+      for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[qb][kb][i] = 0.0f;
+#ifndef SA_DBG_NOQK
+    mma_rows_n<T, D>(s, Kt, 0, qf, lane);
+#endif
+
+    TICK(2)
+    const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
+    Frag pb[QB][KBN][2];
+#ifndef SA_DBG_NOSOFTMAX
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      float mx = -INFINITY;
+      if (interior) {
+#pragma unroll
+        for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) mx = fast_max(mx, s[qb][kb][i]);
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = k0 + kb * 32 + crow(i, h);
+            mx = (key >= lo[qb] && key < hi[qb]) ? fast_max(mx, s[qb][kb][i]) : mx;
+          }
+      }
+      mx = half_max(mx) * sl2e;
+      const bool move = mx > m_run[qb] + kRescaleGap;
+      if (__builtin_amdgcn_ballot_w64(move) != 0) {
+        const float alpha = move ? fast_exp2(m_run[qb] - mx) : 1.0f;
+        m_run[qb] = move ? mx : m_run[qb];
+        l_run[qb] *= alpha;
+#pragma unroll
+        for (int m = 0; m < DB; ++m)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) oacc[qb][m][i] *= alpha;
+      }
+      const float m_use = m_run[qb] == -INFINITY ? 0.0f : m_run[qb];
+#pragma unroll
+      for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[qb][kb][i] = fast_exp2(__builtin_fmaf(s[qb][kb][i], sl2e, -m_use));
+      if (!interior) {
+#pragma unroll
+        for (int kb = 0; kb < KBN; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = k0 + kb * 32 + crow(i, h);
+            s[qb][kb][i] = (key >= lo[qb] && key < hi[qb]) ? s[qb][kb][i] : 0.0f;
+          }
+      }
+      float rs = 0.0f;
+#pragma unroll
+      for (int kb = 0; kb < KBN; ++kb) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) rs += s[qb][kb][i];
+        pack_c<T>(pb[qb][kb], s[qb][kb]);
+      }
+      l_run[qb] += rs;
+    }
+
+#else
+    for (int qb = 0; qb < QB; ++qb) for (int kb = 0; kb < KBN; ++kb) pack_c<T>(pb[qb][kb], s[qb][kb]);
+#endif
+    TICK(3)
+    // O^T[d][q] += V^T P^T
+#pragma unroll
+    for (int kb = 0; kb < KBN; ++kb) {
+      Frag bq[QB][2];
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) bq[qb][0] = pb[qb][kb][0], bq[qb][1] = pb[qb][kb][1];
+#ifndef SA_DBG_NOPV
+      mma_tr_n<T, D>(oacc, Vt, kb, bq, lane);
+      TICK(4)
+#else
+      for (int qb = 0; qb < QB; ++qb) for (int e = 0; e < 8; ++e) oacc[qb][0][e] += (float)bq[qb][0][e] + (float)bq[qb][1][e];
+#endif
+    }
+  }
+
+  // ---- epilogue --------------------------------------------------------------------
+#ifdef SA_DBG_TIMING
+  if (lse_base && lane < 6) {
+    long long tv = lane == 0 ? tacc[0] : lane == 1 ? tacc[1] : lane == 2 ? tacc[2] : lane == 3 ? tacc[3] : lane == 4 ? tacc[4] : tacc[5];
+    m_run[0] = (float)tv / (float)(kt1 - kt0);
+    l_run[0] = 0.5f;
+  }
+#endif
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    const float l_tot = half_sum(l_run[qb]);
+    const bool valid = qrow[qb] < L;
+    if (qrow[qb] < T_) {
+      const float inv = valid ? 1.0f / l_tot : 0.0f;
+      if (!valid) {
+#pragma unroll
+        for (int m = 0; m < DB; ++m)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) oacc[qb][m][i] = 0.0f;
+      }
+      store_acc_T<T, D, DB>(o_base + (int64_t)qrow[qb] * D, oacc[qb], inv, h);
+      if (lse_base && h == 0)
+        lse_base[qrow[qb]] = valid ? m_run[qb] + __builtin_amdgcn_logf(l_tot) : 0.0f;
+    }
   }
 }
 

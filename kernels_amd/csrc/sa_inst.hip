@@ -56,16 +56,29 @@ static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 #if SA_KIND == 0
 template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
-  constexpr int TQ = C::NW * 32;
-  constexpr size_t lds = (size_t)2 * 2 * C::FWD_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
-  auto kern = fwd_kernel<ElemT, D, C::NW, C::FWD_TK>;
-  static std::once_flag once;
-  if (int rc = prepare(kern, lds, once)) return rc;
-  p.n_tiles = (int)ceil_div(p.T, TQ);
-  const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
-  if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
-  return (int)hipGetLastError();
+  if constexpr (C::fwd2(D)) {
+    constexpr int TQ = C::FWD2_NW * C::FWD2_QB * 32;
+    constexpr size_t lds = (size_t)C::FWD2_NST * 2 * C::FWD_TK * D * sizeof(ElemT);
+    auto kern = fwd2_kernel<ElemT, D, C::FWD2_QB, C::FWD2_NW, C::FWD_TK, C::FWD2_NST>;
+    static std::once_flag once;
+    if (int rc = prepare(kern, lds, once)) return rc;
+    p.n_tiles = (int)ceil_div(p.T, TQ);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::FWD2_NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+  } else {
+    constexpr int TQ = C::NW * 32;
+    constexpr size_t lds = (size_t)2 * 2 * C::FWD_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
+    auto kern = fwd_kernel<ElemT, D, C::NW, C::FWD_TK>;
+    static std::once_flag once;
+    if (int rc = prepare(kern, lds, once)) return rc;
+    p.n_tiles = (int)ceil_div(p.T, TQ);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+  }
 }
 template <> int launch_fwd<ElemT, SA_DGROUP>(const FwdParams& p, int D, hipStream_t st) {
 #define X(d) return fwd_d<d>(p, st)
@@ -88,16 +101,29 @@ template <> int launch_delta<ElemT, SA_DGROUP>(const DeltaParams& p, int D, hipS
 }
 template <int D> static int dq_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
-  constexpr int TQ = C::NW * 32;
-  constexpr size_t lds = (size_t)2 * 2 * C::DQ_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
-  auto kern = dq_kernel<ElemT, D, C::NW, C::DQ_TK>;
-  static std::once_flag once;
-  if (int rc = prepare(kern, lds, once)) return rc;
-  p.n_tiles = (int)ceil_div(p.T, TQ);
-  const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
-  if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
-  return (int)hipGetLastError();
+  if constexpr (C::fwd2(D)) {
+    constexpr int TQ = C::DQ2_NW * 32;
+    constexpr size_t lds = (size_t)C::DQ2_NST * 2 * C::DQ2_TK * D * sizeof(ElemT);
+    auto kern = dq2_kernel<ElemT, D, C::DQ2_NW, C::DQ2_TK, C::DQ2_NST>;
+    static std::once_flag once;
+    if (int rc = prepare(kern, lds, once)) return rc;
+    p.n_tiles = (int)ceil_div(p.T, TQ);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::DQ2_NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+  } else {
+    constexpr int TQ = C::NW * 32;
+    constexpr size_t lds = (size_t)2 * 2 * C::DQ_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
+    auto kern = dq_kernel<ElemT, D, C::NW, C::DQ_TK>;
+    static std::once_flag once;
+    if (int rc = prepare(kern, lds, once)) return rc;
+    p.n_tiles = (int)ceil_div(p.T, TQ);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+  }
 }
 template <> int launch_dq<ElemT, SA_DGROUP>(const BwdParams& p, int D, hipStream_t st) {
 #define X(d) return dq_d<d>(p, st)
@@ -107,17 +133,31 @@ template <> int launch_dq<ElemT, SA_DGROUP>(const BwdParams& p, int D, hipStream
 #else
 template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
-  constexpr int TKB = C::NW * 32;
-  constexpr size_t lds =
-      (size_t)2 * (2 * C::DKDV_TQ * TileGeom<ElemT, D>::PITCH * sizeof(ElemT) + 2 * C::DKDV_TQ * sizeof(float));
-  auto kern = dkdv_kernel<ElemT, D, C::NW, C::DKDV_TQ>;
-  static std::once_flag once;
-  if (int rc = prepare(kern, lds, once)) return rc;
-  p.n_tiles = (int)ceil_div(p.T, TKB);
-  const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
-  if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
-  return (int)hipGetLastError();
+  if constexpr (C::fwd2(D)) {
+    constexpr int TKB = C::DKDV2_NW * 32;
+    constexpr size_t lds =
+        (size_t)C::DKDV2_NST * (2 * C::DKDV2_TQ * D * sizeof(ElemT) + 2 * C::DKDV2_TQ * sizeof(float));
+    auto kern = dkdv2_kernel<ElemT, D, C::DKDV2_NW, C::DKDV2_TQ, C::DKDV2_NST>;
+    static std::once_flag once;
+    if (int rc = prepare(kern, lds, once)) return rc;
+    p.n_tiles = (int)ceil_div(p.T, TKB);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::DKDV2_NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+  } else {
+    constexpr int TKB = C::NW * 32;
+    constexpr size_t lds =
+        (size_t)2 * (2 * C::DKDV_TQ * TileGeom<ElemT, D>::PITCH * sizeof(ElemT) + 2 * C::DKDV_TQ * sizeof(float));
+    auto kern = dkdv_kernel<ElemT, D, C::NW, C::DKDV_TQ>;
+    static std::once_flag once;
+    if (int rc = prepare(kern, lds, once)) return rc;
+    p.n_tiles = (int)ceil_div(p.T, TKB);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+  }
 }
 template <> int launch_dkdv<ElemT, SA_DGROUP>(const BwdParams& p, int D, hipStream_t st) {
 #define X(d) return dkdv_d<d>(p, st)

@@ -15,8 +15,46 @@ template <typename T, int DGROUP> int launch_dq(const BwdParams& p, int D, hipSt
 template <typename T, int DGROUP> int launch_dkdv(const BwdParams& p, int D, hipStream_t st);
 
 // tile sizes, shared between the launchers and sa_query()
+#ifndef SA_FWD2_QB
+#define SA_FWD2_QB 1
+#endif
+#ifndef SA_DQ2_NW
+#define SA_DQ2_NW 8
+#endif
+#ifndef SA_DQ2_TK
+#define SA_DQ2_TK 64
+#endif
+#ifndef SA_DQ2_NST
+#define SA_DQ2_NST 2
+#endif
+#ifndef SA_DKDV2_NW
+#define SA_DKDV2_NW 4
+#endif
+#ifndef SA_DKDV2_TQ
+#define SA_DKDV2_TQ 64
+#endif
+#ifndef SA_DKDV2_NST
+#define SA_DKDV2_NST 2
+#endif
+#ifndef SA_FWD2_NW
+#define SA_FWD2_NW 8
+#endif
+#ifndef SA_FWD2_NST
+#define SA_FWD2_NST 2
+#endif
 template <typename T> struct Cfg {
   static constexpr int NW = 4;                                   // waves per workgroup
+  // 16-bit, D in {64, 128}: forward kernel with QB query blocks per wave and NST LDS stages
+  static constexpr int FWD2_NW = SA_FWD2_NW;
+  static constexpr int DQ2_NW = SA_DQ2_NW, DQ2_TK = SA_DQ2_TK, DQ2_NST = SA_DQ2_NST;
+  static constexpr int DKDV2_NW = SA_DKDV2_NW, DKDV2_TQ = SA_DKDV2_TQ, DKDV2_NST = SA_DKDV2_NST;
+  static constexpr int FWD2_QB = SA_FWD2_QB;
+  static constexpr int FWD2_NST = SA_FWD2_NST;
+#ifdef SA_FWD2_DISABLE
+  static constexpr bool fwd2(int) { return false; }
+#else
+  static constexpr bool fwd2(int D) { return sizeof(T) == 2 && (D == 64 || D == 128); }
+#endif
   static constexpr int FWD_TK = sizeof(T) == 4 ? 32 : 64;        // keys per forward step
   static constexpr int DQ_TK = 32;                               // keys per dQ step
   static constexpr int DKDV_TQ = 32;                             // queries per dK/dV step
