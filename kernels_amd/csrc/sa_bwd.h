@@ -14,6 +14,7 @@
 // query tiles that can see those keys (kernel.py:1046-1054).  Both kernels write every
 // element of their outputs, zeros included, so the caller does not pre-clear them.
 #pragma once
+#include <type_traits>
 #include "sa_common.h"
 
 namespace sa {
@@ -435,10 +436,15 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
 
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh;
   const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh;
-  auto issue_tile = [&](int t) {
+  Loader ldk, ldv;
+  ldk.init(kbase, p.k_st, kt0 * TK, T_ - 1, wave, lane);
+  ldv.init(vbase, p.v_st, kt0 * TK, T_ - 1, wave, lane);
+  auto issue_tile = [&](int t) {   // tiles are issued in ascending order
     T* st = smem + ((t - kt0) % NST) * STAGE;
-    Loader::issue(kbase, p.k_st, t * TK, T_ - 1, st, wave, lane);
-    Loader::issue(vbase, p.v_st, t * TK, T_ - 1, st + TILE, wave, lane);
+    ldk.issue(st, wave);
+    ldv.issue(st + TILE, wave);
+    ldk.advance();
+    ldv.advance();
   };
 #pragma unroll
   for (int i = 0; i < NST - 1; ++i)
@@ -579,10 +585,11 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
   const float* lse_base = p.lse + (int64_t)bh * T_;
   const float* delta_base = p.delta + (int64_t)bh * T_;
   auto stage_ptr = [&](int t) { return smem_raw + ((t - qt0) % NST) * STAGE_BYTES; };
-  auto issue_tile = [&](int t) {
+  Loader ldq, ldg;
+  ldq.init(qbase, p.q_st, qt0 * TQ, T_ - 1, wave, lane);
+  ldg.init(gbase, p.do_st, qt0 * TQ, T_ - 1, wave, lane);
+  auto issue_tile = [&](int t) {   // tiles are issued in ascending order
     T* st = reinterpret_cast<T*>(stage_ptr(t));
-    Loader::issue(qbase, p.q_st, t * TQ, T_ - 1, st, wave, lane);
-    Loader::issue(gbase, p.do_st, t * TQ, T_ - 1, st + TILE, wave, lane);
     // lanes [0, RPW) fetch lse, lanes [RPW, 2*RPW) fetch delta of this wave's RPW rows
     if (lane < 2 * RPW) {
       int r = t * TQ + wave * RPW + (lane % RPW);
@@ -592,6 +599,10 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                        (SA_LDS void*)dst, 4, 0, 0);
     }
+    ldq.issue(st, wave);
+    ldg.issue(st + TILE, wave);
+    ldq.advance();
+    ldg.advance();
   };
 #pragma unroll
   for (int i = 0; i < NST - 1; ++i)
@@ -619,11 +630,20 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
     for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
   wait_all_loads();
 
+#ifdef SA_DBG_TIMING
+  long long tacc[6] = {0,0,0,0,0,0}; long long tp = __builtin_readcyclecounter();
+#define TICK(i) { long long tn = __builtin_readcyclecounter(); tacc[i] += tn - tp; tp = tn; }
+#else
+#define TICK(i)
+#endif
   for (int t = qt0; t < qt1; ++t) {
     if (NST == 3 && t + 1 < qt1) wait_loads<LPT>();
     else wait_loads<0>();
+    TICK(0)
     __syncthreads();
+    TICK(1)
     if (t + NST - 1 < qt1) issue_tile(t + NST - 1);
+    TICK(2)
 
     const T* Qt = reinterpret_cast<const T*>(stage_ptr(t));
     const T* Gt = Qt + TILE;
@@ -636,20 +656,27 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
       f32x16 s[1], dp[1];
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[0][i] = 0.0f, dp[0][i] = 0.0f;
-      mma_rows<T, D>(s, Qt, qb * 32, kf, lane);    // S[q][key] = Q K^T
-      mma_rows<T, D>(dp, Gt, qb * 32, vf, lane);   // dP[q][key] = dO V^T
+      // lse / delta of the 16 rows this lane holds: fetched ahead of the products so that
+      // their LDS latency is not exposed in the element-wise phase
+      f32x4 l4[4], d4[4];
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         const int r = qb * 32 + 8 * g4 + 4 * h;     // tile row of 4 consecutive C-fragment rows
         const float* chunk = ld_t + (r / RPW) * 2 * RPW + (r % RPW);
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(chunk);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(chunk + RPW);
+        l4[g4] = *reinterpret_cast<const f32x4*>(chunk);
+        d4[g4] = *reinterpret_cast<const f32x4*>(chunk + RPW);
+      }
+      mma_rows<T, D>(s, Qt, qb * 32, kf, lane);    // S[q][key] = Q K^T
+      mma_rows<T, D>(dp, Gt, qb * 32, vf, lane);   // dP[q][key] = dO V^T
+      TICK(3)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int i = 4 * g4 + e;
-          const float pr = fast_exp2(__builtin_fmaf(s[0][i], sl2e, -l4[e]));
+          const float pr = fast_exp2(__builtin_fmaf(s[0][i], sl2e, -l4[g4][e]));
           s[0][i] = pr;
-          dp[0][i] = pr * (dp[0][i] - d4[e]);
+          dp[0][i] = pr * (dp[0][i] - d4[g4][e]);
         }
       }
       if (!interior) {
@@ -661,11 +688,19 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
           dp[0][i] = ok ? dp[0][i] : 0.0f;
         }
       }
+      TICK(4)
       mma_tr<T, D>(dv, Gt, qb, s[0], lane);    // dV^T[d][key] += dO^T P
       mma_tr<T, D>(dk, Qt, qb, dp[0], lane);   // dK^T[d][key] += Q^T dS
+      TICK(5)
     }
   }
 
+#ifdef SA_DBG_TIMING
+  if (lane < 6 && krow < T_) {
+    long long tv = lane == 0 ? tacc[0] : lane == 1 ? tacc[1] : lane == 2 ? tacc[2] : lane == 3 ? tacc[3] : lane == 4 ? tacc[4] : tacc[5];
+    dv[0][0] = (float)tv / (float)(qt1 - qt0);
+  }
+#endif
   if (krow < T_) {
     if (krow >= L) {
 #pragma unroll

@@ -308,12 +308,18 @@ SA_DEV void mma_tr_n(f32x16 (&acc)[NQ][NM], const T* X, int rb, const typename E
       });
 }
 
-// Asynchronous copy of a [ROWS][D] row-major global tile into a swizzled LDS tile with
+// Asynchronous copy of [ROWS][D] row-major global tiles into swizzled LDS tiles with
 // global_load_lds_dwordx4: the data never passes through registers.  One instruction moves
 // 1 KiB (64 lanes x 16 bytes) to consecutive LDS addresses, i.e. 1024/(2*D) whole rows; lane l
 // therefore fetches, for physical chunk l % CPR of its row, the logical chunk that the swizzle
 // maps there.  The NW waves of a workgroup interleave instruction by instruction.  Completion
 // is tracked by vmcnt; visibility to the other waves needs a barrier after the wait.
+//
+// Tiles are issued in ascending order.  The object keeps, per lane, the 32-bit element offset
+// of its row in the next tile, so that issuing costs an add, a clamp and an add per
+// instruction and no multiplication; rows past the end of the sequence are clamped to the
+// last row (their contents are masked by the caller).  Offsets are 32-bit: the host checks
+// that T * row_stride fits.
 template <typename T, int D, int ROWS, int NW> struct AsyncTile {
   using G_ = TileGeom<T, D>;
   static_assert(G_::SWZ, "asynchronous tiles use the swizzled layout");
@@ -321,39 +327,41 @@ template <typename T, int D, int ROWS, int NW> struct AsyncTile {
   static constexpr int RPI = 1024 / ROW_BYTES;             // rows per instruction
   static constexpr int NI = ROWS / RPI;                     // instructions per tile
   static_assert(ROWS % (RPI * NW) == 0, "tile must split evenly over the waves");
+  static_assert((RPI * NW) % 16 == 0, "the swizzle of a lane must not depend on the instruction");
   static constexpr int PER_WAVE = NI / NW;                  // instructions per wave per tile
 
-  // Issue this wave's share of the tile whose first row is row0 (rows clamped to last_row).
-  // The address of a lane is (wave-uniform 64-bit row base) + (32-bit lane offset): the
-  // uniform part is scalar arithmetic, and the lane offset does not change from tile to tile
-  // unless the tile hangs over the end of the sequence.
-  SA_DEV static void issue(const T* gbase, int64_t row_stride, int row0, int last_row, T* tile, int wave,
-                           int lane) {
+  const T* base;      // wave-uniform: first element of this (batch, head)
+  uint32_t rowoff;    // element offset of this lane's row (instruction 0) in the next tile
+  uint32_t coloff;    // swizzled column offset of this lane, in elements
+  uint32_t last;      // element offset of the last valid row
+  uint32_t istep;     // offset between rows of consecutive instructions of one wave
+  uint32_t tstep;     // offset between consecutive tiles
+
+  SA_DEV void init(const T* gbase, int64_t row_stride, int first_row, int last_row, int wave, int lane) {
     const int lrow = lane / G_::CPR, pch = lane % G_::CPR;
     const uint32_t rs = (uint32_t)row_stride;
-    if (row0 + ROWS - 1 <= last_row) {
+    base = gbase;
+    rowoff = (uint32_t)(first_row + wave * RPI + lrow) * rs;
+    coloff = (uint32_t)((pch ^ G_::swz(wave * RPI + lrow)) * Elem<T>::VEC);
+    last = (uint32_t)last_row * rs;
+    istep = (uint32_t)(NW * RPI) * rs;
+    tstep = (uint32_t)ROWS * rs;
+  }
+  // instructions [I0, I1) of this wave's share of the next tile
+  template <int I0, int I1> SA_DEV void issue_part(T* tile, int wave) const {
+    static_assert(0 <= I0 && I0 <= I1 && I1 <= PER_WAVE, "instruction range");
 #pragma unroll
-      for (int i = 0; i < PER_WAVE; ++i) {
-        const int rb = (i * NW + wave) * RPI;                // wave-uniform first row of this instruction
-        const uint32_t loff = (uint32_t)lrow * rs + (uint32_t)((pch ^ G_::swz(rb + lrow)) * Elem<T>::VEC);
-        const T* src = gbase + (int64_t)(row0 + rb) * row_stride + loff;
-        T* dst = tile + rb * D;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (SA_LDS void*)dst, 16, 0, 0);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < PER_WAVE; ++i) {
-        const int rb = (i * NW + wave) * RPI;
-        int gr = row0 + rb + lrow;
-        gr = gr < last_row ? gr : last_row;
-        const T* src = gbase + (int64_t)gr * row_stride + ((pch ^ G_::swz(rb + lrow)) * Elem<T>::VEC);
-        T* dst = tile + rb * D;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (SA_LDS void*)dst, 16, 0, 0);
-      }
+    for (int i = I0; i < I1; ++i) {
+      uint32_t ro = rowoff + (uint32_t)i * istep;
+      ro = ro < last ? ro : last;
+      const T* src = base + (ro + coloff);
+      T* dst = tile + (i * NW + wave) * RPI * D;           // wave-uniform
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (SA_LDS void*)dst, 16, 0, 0);
     }
   }
+  SA_DEV void issue(T* tile, int wave) const { issue_part<0, PER_WAVE>(tile, wave); }
+  SA_DEV void advance() { rowoff += tstep; }
 };
 
 // s_waitcnt vmcnt(N), other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and 15:14).

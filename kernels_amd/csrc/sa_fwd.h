@@ -303,10 +303,15 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
 
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh;
   const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh;
-  auto issue_tile = [&](int t) {
+  Loader ldk, ldv;
+  ldk.init(kbase, p.k_st, kt0 * TK, T_ - 1, wave, lane);
+  ldv.init(vbase, p.v_st, kt0 * TK, T_ - 1, wave, lane);
+  auto issue_tile = [&](int t) {   // tiles are issued in ascending order
     T* st = smem + ((t - kt0) % NST) * STAGE;
-    Loader::issue(kbase, p.k_st, t * TK, T_ - 1, st, wave, lane);
-    Loader::issue(vbase, p.v_st, t * TK, T_ - 1, st + TILE, wave, lane);
+    ldk.issue(st, wave);
+    ldv.issue(st + TILE, wave);
+    ldk.advance();
+    ldv.advance();
   };
   // prologue: NST-1 tiles in flight
 #pragma unroll
