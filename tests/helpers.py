@@ -1,0 +1,41 @@
+"""Shared helpers for the test-suite: seeded inputs the way the reference's own test builds
+them (tests/test_streaming_attention.py:78-150) and the comparison bars."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+# parity bars: fp32 <= 1e-4 abs; bf16/fp16 <= 2e-2 abs + 1e-2 rel against the fp32/f64 oracle
+TOL = {torch.float32: (1e-4, 0.0), torch.float16: (2e-2, 1e-2), torch.bfloat16: (2e-2, 1e-2)}
+
+
+def make_inputs(B, H, T, D, seed=20, dtype=torch.float32):
+    """q, k, v, dO ~ N(0,1) from a seeded CPU generator, rounded to ``dtype`` (the values the
+    kernel will actually see), returned as CPU tensors of that dtype."""
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(B, H, T, D, generator=g).to(dtype) for _ in range(4)]
+
+
+def tricky_lens(B, T, C, R, seed=20):
+    """Lengths around the chunk size, the window size, T and T+1 (> T must clamp), as in
+    tests/test_streaming_attention.py:117-135 but drawn from a seeded generator."""
+    cand = [2, 5, C, C + 1, max(C - 1, 1), max(C // 2, 1), C // 2 + C, max(C * R, 1), C * R + 1,
+            max(C * R - 1, 1), T + 1, T, max(T // 2, 1), max(T // 4, 1)]
+    cand = [min(max(int(x), 1), 2**31 - 1) for x in cand]
+    rng = np.random.default_rng(seed)
+    return torch.tensor(rng.choice(cand, B), dtype=torch.int32)
+
+
+def assert_close(name, got, want, dtype):
+    atol, rtol = TOL[dtype]
+    got = torch.as_tensor(got).detach().double().cpu()
+    want = torch.as_tensor(want).detach().double().cpu()
+    assert got.shape == want.shape, f"{name}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got).all(), f"{name}: non-finite values"
+    err = (got - want).abs()
+    bound = atol + rtol * want.abs()
+    bad = err > bound
+    assert not bad.any(), (
+        f"{name}: {int(bad.sum())} elements out of tolerance, max abs err {err.max().item():.3e} "
+        f"(atol {atol}, rtol {rtol}), worst at {np.unravel_index(int(err.argmax()), err.shape)}"
+    )

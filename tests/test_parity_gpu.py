@@ -1,0 +1,320 @@
+"""Parity of the HIP path against the oracle, on a real MI355X.
+
+Every call goes through the public API / dispatcher ops, which reach the kernels only
+through the C ABI of libstreaming_attention.so.  Bars: fp32 <= 1e-4 abs; bf16/fp16 <= 2e-2 abs
++ 1e-2 rel, against the float64 (small shapes) or fp32 windowed (full-size shapes) oracle."""
+import ctypes
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import sa_oracle
+from tests.helpers import TOL, assert_close, make_inputs, tricky_lens
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "streaming_attention_small.npz")
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _library_loaded():
+    from streaming_attention import _lib
+
+    _lib.load()   # fail loudly here rather than silently somewhere else
+    os.environ.setdefault("STREAMING_ATTENTION_EAGER", "1")
+    yield
+
+
+def run_kernel(q, k, v, d_o, lens, C, R, **kw):
+    """CPU tensors in, CPU tensors out; forward + backward on cuda:0."""
+    from streaming_attention import streaming_attention
+
+    dev = torch.device("cuda:0")
+    qd, kd, vd = (t.to(dev).requires_grad_() for t in (q, k, v))
+    ld = lens.to(dev) if lens is not None else None
+    out, lse = streaming_attention(qd, kd, vd, ld, C, R, return_lse=True, **kw)
+    out.backward(d_o.to(dev))
+    torch.cuda.synchronize()
+    return out.detach().cpu(), lse.detach().cpu(), qd.grad.cpu(), kd.grad.cpu(), vd.grad.cpu()
+
+
+def check_against_dense(q, k, v, d_o, lens, C, R, dtype, **kw):
+    o, lse, dq, dk, dv = run_kernel(q, k, v, d_o, lens, C, R, **kw)
+    ref = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=kw.get("sm_scale"), d_out=d_o)
+    assert_close("O", o, ref["O"], dtype)
+    assert_close("dQ", dq, ref["dQ"], dtype)
+    assert_close("dK", dk, ref["dK"], dtype)
+    assert_close("dV", dv, ref["dV"], dtype)
+    assert_close("LSE", lse, ref["LSE"], torch.float32 if dtype == torch.float32 else dtype)
+    B, T = q.shape[0], q.shape[2]
+    L = sa_oracle.clamp_lens(lens, B, T)
+    for b in range(B):   # exact zeros at padded positions, as the reference's zeros_like gives
+        for t in (o, dq, dk, dv):
+            assert not t[b, :, int(L[b]):].any()
+    return o, lse, dq, dk, dv
+
+
+SHAPES = [(1, 1, 1), (5, 3, 10), (1, 6, 16), (5, 3, 800)]
+WINDOWS = [(1, 0), (1, 5), (10, 0), (10, 5), (10, 10000), (32, 5), (10000, 0), (10000, 10000)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("D", [16, 64])
+@pytest.mark.parametrize("lens_mode", ["none", "tricky"])
+@pytest.mark.parametrize("C,R", WINDOWS)
+@pytest.mark.parametrize("B,H,T", SHAPES)
+def test_reference_grid(B, H, T, D, C, R, lens_mode, dtype):
+    """The reference's own grid (tests/test_streaming_attention.py:11-31), reduced."""
+    q, k, v, d_o = make_inputs(B, H, T, D, dtype=dtype)
+    lens = tricky_lens(B, T, C, R) if lens_mode == "tricky" else None
+    check_against_dense(q, k, v, d_o, lens, C, R, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("D", [16, 32, 64, 128, 256])
+def test_all_head_dims(D, dtype):
+    B, H, T, C, R = 2, 2, 200, 16, 2
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=21, dtype=dtype)
+    lens = torch.tensor([T, 77], dtype=torch.int32)
+    check_against_dense(q, k, v, d_o, lens, C, R, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("T,C,R", [(257, 64, 2), (513, 128, 1), (300, 256, 8), (1000, 96, 3), (640, 32, 20)])
+def test_tile_edges_16bit(T, C, R, dtype):
+    """Lengths and chunk sizes that straddle the kernels' 32/64/128/256-wide tiles."""
+    B, H, D = 2, 2, 128
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=22, dtype=dtype)
+    lens = torch.tensor([T, max(1, T - 65)], dtype=torch.int32)
+    check_against_dense(q, k, v, d_o, lens, C, R, dtype)
+
+
+def test_golden_vectors():
+    data = np.load(GOLDEN, allow_pickle=False)
+    for name in sorted({k.split(".")[0] for k in data.files}):
+        B, H, T, D, C, R = data[f"{name}.shape"].tolist()
+        lens = data[f"{name}.lens"]
+        lt = None if lens[0] < 0 else torch.from_numpy(lens)
+        q, k, v, d_o = (torch.from_numpy(data[f"{name}.{x}"]).float() for x in ("q", "k", "v", "d_o"))
+        o, _, dq, dk, dv = run_kernel(q, k, v, d_o, lt, C, R)
+        for key, got in (("o", o), ("dq", dq), ("dk", dk), ("dv", dv)):
+            assert_close(f"{name}.{key}", got, data[f"{name}.{key}"], torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=str)
+def test_noncontiguous_inputs(dtype):
+    """[B,T,H,D]-stored q/k/v (read in place), sliced views (copied by the host), a strided
+    int32 lens and a strided fp32 upstream gradient."""
+    from streaming_attention import streaming_attention
+
+    dev = torch.device("cuda:0")
+    B, H, T, D, C, R = 3, 2, 70, 64, 16, 1
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=23, dtype=dtype)
+    lens = torch.tensor([70, 33, 71], dtype=torch.int32)
+    ref = sa_oracle.dense_f64(q, k, v, lens, C, R, d_out=d_o)
+
+    def variants(t):
+        bthd = t.to(dev).transpose(1, 2).contiguous().transpose(1, 2)
+        big = torch.zeros(B, H, T, 2 * D, dtype=dtype, device=dev)
+        big[..., 1::2] = t.to(dev)
+        return bthd, big[..., 1::2]
+
+    lens_big = torch.zeros(2 * B, dtype=torch.int32, device=dev)
+    lens_big[::2] = lens.to(dev)
+    for which in (0, 1):
+        qd, kd, vd = (variants(t)[which].detach().requires_grad_() for t in (q, k, v))
+        assert not qd.is_contiguous()
+        out = streaming_attention(qd, kd, vd, lens_big[::2], C, R)
+        g32 = torch.zeros(B, H, T, 2 * D, dtype=torch.float32, device=dev)
+        g32[..., ::2] = d_o.to(dev).float()
+        out.backward(g32[..., ::2].to(out.dtype) if which == 0 else variants(d_o)[1])
+        assert out.is_contiguous()
+        assert_close("O", out, ref["O"], dtype)
+        assert_close("dQ", qd.grad, ref["dQ"], dtype)
+        assert_close("dK", kd.grad, ref["dK"], dtype)
+        assert_close("dV", vd.grad, ref["dV"], dtype)
+
+
+def test_backward_op_accepts_foreign_gradient_and_missing_lse():
+    """The backward dispatcher op on its own: fp32 strided dO with fp16 q/k/v
+    (tests/test_streaming_attention.py:224-248) and an empty lse (forward without return_lse)."""
+    dev = torch.device("cuda:0")
+    B, H, T, D, C, R = 2, 2, 90, 64, 10, 3
+    dtype = torch.float16
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=24, dtype=dtype)
+    lens = torch.tensor([90, 41], dtype=torch.int32)
+    qd, kd, vd = (t.to(dev) for t in (q, k, v))
+    fwd = torch.ops.alexdremov_streaming_attention.forward
+    bwd = torch.ops.alexdremov_streaming_attention.backward
+    o, lse = fwd(qd, kd, vd, lens.to(dev), C, R, D ** -0.5, False, False, False, "ieee")
+    assert lse.numel() == 0 and lse.device.type == "cpu"
+    g = torch.zeros(B, H, T, 2 * D, dtype=torch.float32, device=dev)
+    g[..., ::2] = d_o.to(dev).float()
+    dq, dk, dv = bwd(qd, kd, vd, lens.to(dev), o, lse, g[..., ::2], C, R, D ** -0.5, False, False, "ieee")
+    ref = sa_oracle.dense_f64(q, k, v, lens, C, R, d_out=d_o)
+    assert_close("dQ", dq, ref["dQ"], dtype)
+    assert_close("dK", dk, ref["dK"], dtype)
+    assert_close("dV", dv, ref["dV"], dtype)
+
+
+@pytest.mark.parametrize("scale", [0.37, -0.2, 0.0])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=str)
+def test_softmax_scale(scale, dtype):
+    """Explicit, negative and zero softmax scales.  For bf16 the large scale is halved: with
+    N(0,1) inputs a scale of 0.37 at D=64 gives gradients of magnitude ~5, whose bf16 rounding
+    alone exceeds the absolute part of the bar."""
+    if dtype == torch.bfloat16 and scale > 0.2:
+        scale = 0.18
+    B, H, T, D, C, R = 2, 2, 100, 64, 32, 1
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=25, dtype=dtype)
+    lens = torch.tensor([100, 64], dtype=torch.int32)
+    check_against_dense(q, k, v, d_o, lens, C, R, dtype, sm_scale=scale)
+
+
+def test_empty_inputs_and_zero_lengths():
+    from streaming_attention import streaming_attention
+
+    dev = torch.device("cuda:0")
+    for shape in ((0, 2, 8, 64), (2, 2, 0, 64)):
+        q = torch.zeros(shape, device=dev, requires_grad=True)
+        out = streaming_attention(q, q, q, None, 4, 1)
+        assert out.shape == q.shape
+    q, k, v, d_o = make_inputs(2, 2, 40, 64, seed=26)
+    lens = torch.tensor([0, 40], dtype=torch.int32)
+    o, lse, dq, dk, dv = check_against_dense(q, k, v, d_o, lens, 8, 1, torch.float32)
+    assert not o[0].any() and not dq[0].any()
+
+
+def test_c_abi_direct_calls():
+    """ctypes straight into the shared library, no dispatcher in between."""
+    from streaming_attention import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    B, H, T, D, C, R = 2, 3, 150, 128, 32, 2
+    dtype = torch.bfloat16
+    q, k, v, d_o = (t.to(dev) for t in make_inputs(B, H, T, D, seed=27, dtype=dtype))
+    lens = torch.tensor([150, 99], dtype=torch.int32, device=dev)
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, T, dtype=torch.float32, device=dev)
+    delta = torch.empty_like(lse)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    s4 = _lib.strides4
+    st = torch.cuda.current_stream().cuda_stream
+    sc = D ** -0.5
+    assert lib.sa_forward(q.data_ptr(), k.data_ptr(), v.data_ptr(), lens.data_ptr(), 1, o.data_ptr(), lse.data_ptr(),
+                          s4(q), s4(k), s4(v), B, H, T, D, C, R, sc, 2, st) == 0
+    assert lib.sa_bwd_delta(o.data_ptr(), d_o.data_ptr(), delta.data_ptr(), s4(o), s4(d_o), B, H, T, D, 2, st) == 0
+    assert lib.sa_bwd_dq(q.data_ptr(), k.data_ptr(), v.data_ptr(), lens.data_ptr(), 1, d_o.data_ptr(), lse.data_ptr(),
+                         delta.data_ptr(), dq.data_ptr(), s4(q), s4(k), s4(v), s4(d_o), B, H, T, D, C, R, sc, 2, st) == 0
+    assert lib.sa_bwd_dkdv(q.data_ptr(), k.data_ptr(), v.data_ptr(), lens.data_ptr(), 1, d_o.data_ptr(),
+                           lse.data_ptr(), delta.data_ptr(), dk.data_ptr(), dv.data_ptr(), s4(q), s4(k), s4(v),
+                           s4(d_o), B, H, T, D, C, R, sc, 2, st) == 0
+    torch.cuda.synchronize()
+    ref = sa_oracle.dense_f64(q.cpu(), k.cpu(), v.cpu(), lens.cpu(), C, R, d_out=d_o.cpu())
+    for name, got in (("O", o), ("dQ", dq), ("dK", dk), ("dV", dv)):
+        assert_close(name, got, ref[name], dtype)
+    want_delta = (ref["O"] * d_o.double().cpu().numpy()).sum(-1)
+    assert_close("delta", delta, want_delta, dtype)
+    # sa_backward = the three launches behind one entry point
+    dq2, dk2, dv2 = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    assert lib.sa_backward(q.data_ptr(), k.data_ptr(), v.data_ptr(), lens.data_ptr(), 1, o.data_ptr(), d_o.data_ptr(),
+                           lse.data_ptr(), delta.data_ptr(), dq2.data_ptr(), dk2.data_ptr(), dv2.data_ptr(),
+                           s4(q), s4(k), s4(v), s4(o), s4(d_o), B, H, T, D, C, R, sc, 2, st) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+    # a layout the kernels cannot read in place is refused, not mis-read
+    assert lib.sa_forward(q.data_ptr() + 2, k.data_ptr(), v.data_ptr(), None, 0, o.data_ptr(), None,
+                          s4(q), s4(k), s4(v), B, H, T, D, C, R, sc, 2, st) == -4
+
+
+# ---- BASELINE.json configurations at their real shapes -------------------------------
+
+def _lens_for(mode, B, T, g):
+    if mode == "full":
+        return None
+    if mode == "uniform_half_full":
+        return torch.randint(T // 2, T + 1, (B,), generator=g, dtype=torch.int32)
+    if mode == "uniform_256_512":
+        return torch.randint(256, 513, (B,), generator=g, dtype=torch.int32)
+    u = torch.rand(B, generator=g, dtype=torch.float64)
+    return torch.exp(math.log(64.0) + u * (math.log(T) - math.log(64.0))).round().to(torch.int32)
+
+
+CONFIGS = [
+    ("cfg2_bf16_T4096_D64", 8, 16, 4096, 64, torch.bfloat16, 128, 4, "full", None),
+    ("cfg3_headline_bf16_T16384_D128", 4, 16, 16384, 128, torch.bfloat16, 256, 8, "uniform_half_full", 1.0),
+    ("cfg4_ragged_fp16_T2048_D128", 16, 8, 2048, 128, torch.float16, 64, 1, "loguniform", 1.0),
+    ("cfg5_long_bf16_T65536_D128", 1, 32, 65536, 128, torch.bfloat16, 512, 16, "full", 1.0),
+]
+
+
+def test_baseline_config1_fp32():
+    B, H, T, D, C, R = 2, 4, 512, 64, 64, 2
+    g = torch.Generator().manual_seed(20)
+    q, k, v, d_o = [torch.randn(B, H, T, D, generator=g) for _ in range(4)]
+    lens = torch.randint(256, 513, (B,), generator=g, dtype=torch.int32)
+    check_against_dense(q, k, v, d_o, lens, C, R, torch.float32)
+    # and against the reference's own formulation (mask + SDPA, fp32)
+    o, _, dq, dk, dv = run_kernel(q, k, v, d_o, lens, C, R)
+    ro, rdq, rdk, rdv = sa_oracle.sdpa_fwd_bwd(q, k, v, lens, C, R, d_o)
+    for name, a, b in (("O", o, ro), ("dQ", dq, rdq), ("dK", dk, rdk), ("dV", dv, rdv)):
+        assert_close(name, a, b, torch.float32)
+
+
+@pytest.mark.parametrize("name,B,H,T,D,dtype,C,R,lens_mode,qkv_scale", CONFIGS, ids=[c[0] for c in CONFIGS])
+def test_baseline_configs_full_size(name, B, H, T, D, dtype, C, R, lens_mode, qkv_scale):
+    """Full-size shapes against the windowed fp32 oracle evaluated on the GPU with torch
+    matmuls (a dense T x T mask does not fit), plus size-independent properties."""
+    from streaming_attention import streaming_attention
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(20)
+    lens = _lens_for(lens_mode, B, T, g)
+    dg = torch.Generator(device=dev).manual_seed(20)
+    sc = D ** -0.5 if qkv_scale is None else qkv_scale
+    q, k, v = [(torch.randn(B, H, T, D, generator=dg, device=dev) * sc).to(dtype).requires_grad_() for _ in range(3)]
+    d_o = torch.randn(B, H, T, D, generator=dg, device=dev).to(dtype)
+    ld = lens.to(dev) if lens is not None else None
+    out, lse = streaming_attention(q, k, v, ld, C, R, return_lse=True)
+    out.backward(d_o)
+    torch.cuda.synchronize()
+    ro, rlse, rdq, rdk, rdv = sa_oracle.windowed(q, k, v, lens, C, R, d_out=d_o)
+    for nm, a, b in (("O", out, ro), ("dQ", q.grad, rdq), ("dK", k.grad, rdk), ("dV", v.grad, rdv), ("LSE", lse, rlse)):
+        atol, rtol = TOL[dtype]
+        err = (a.detach().float() - b).abs()
+        bound = atol + rtol * b.abs()
+        assert bool((err <= bound).all()), f"{name} {nm}: max err {err.max().item():.3e}"
+        assert bool(torch.isfinite(a).all())
+    L = sa_oracle.clamp_lens(lens, B, T)
+    for b in range(B):
+        for t in (out, q.grad, k.grad, v.grad):
+            assert not bool(t[b, :, int(L[b]):].any()), "padded positions must be exactly zero"
+    # determinism: the kernels use no atomics, a second run is bit-identical
+    q2, k2, v2 = (t.detach().clone().requires_grad_() for t in (q, k, v))
+    out2 = streaming_attention(q2, k2, v2, ld, C, R)
+    out2.backward(d_o)
+    assert torch.equal(out, out2) and torch.equal(q.grad, q2.grad) and torch.equal(k.grad, k2.grad)
+    assert torch.equal(v.grad, v2.grad)
+    if B > 1:
+        # batch entries are independent: reversing the batch reverses the outputs bit for bit
+        perm = torch.arange(B - 1, -1, -1, device=dev)
+        q3, k3, v3 = (t.detach()[perm].clone().requires_grad_() for t in (q, k, v))
+        out3 = streaming_attention(q3, k3, v3, ld[perm] if ld is not None else None, C, R)
+        out3.backward(d_o[perm])
+        assert torch.equal(out3, out[perm]) and torch.equal(q3.grad, q.grad[perm])
+        assert torch.equal(k3.grad, k.grad[perm]) and torch.equal(v3.grad, v.grad[perm])
+    if lens is not None:
+        # a sequence of length L equals the same sequence cut to L positions
+        b = int(np.argmin(L))
+        Lb = int(L[b])
+        q4, k4, v4 = (t.detach()[b:b + 1, :, :Lb].clone().requires_grad_() for t in (q, k, v))
+        out4 = streaming_attention(q4, k4, v4, None, C, R)
+        out4.backward(d_o[b:b + 1, :, :Lb])
+        for a, bb in ((out4, out[b:b + 1, :, :Lb]), (q4.grad, q.grad[b:b + 1, :, :Lb]),
+                      (k4.grad, k.grad[b:b + 1, :, :Lb]), (v4.grad, v.grad[b:b + 1, :, :Lb])):
+            assert torch.allclose(a.float(), bb.float(), atol=1e-3, rtol=1e-3)
