@@ -166,6 +166,8 @@ def main():
     ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel-iters", type=int, default=10)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a 1 GiB device-to-device copy (known traffic) for scaling HBM counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -175,6 +177,14 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB read + 1 GiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "3 copies of 1 GiB (2^28 fp32): 1048576 KiB read and written each"}))
+        return
     w = make_inputs(args.workload, dev)
     B, H, T, D, C, R = w["B"], w["H"], w["T"], w["D"], w["C"], w["R"]
     P = unmasked_pairs(T, C, R, w["lens_list"])
