@@ -406,13 +406,27 @@ template <typename T, int D, int ROWS, int NT> struct Stager {
   }
 };
 
-// Hardware hands workgroup i to XCD i % 8.  Renumber so that each XCD receives a
-// contiguous range of logical ids: neighbouring tiles of one (batch, head) then share
-// that XCD's L2 for the keys and values they have in common.
-SA_DEV int xcd_remap(int bid, int n) {
-  const int per = n >> 3, rem = n & 7;
-  const int x = bid & 7, idx = bid >> 3;
-  return x * per + (x < rem ? x : rem) + idx;
+// Hardware hands workgroup i to XCD i % 8 (each XCD has its own L2).  Map block ids so that
+// all tiles of one (batch, head) run on one XCD, in consecutive dispatch slots -- neighbouring
+// tiles then share that L2 for the keys and values they have in common -- and so that the
+// (batch, head) pairs are dealt round-robin over the XCDs: with ragged sequence lengths every
+// XCD then receives a mix of long and short batches instead of a contiguous block of one.
+// Tiles are visited from the end of the sequence backwards: the long-window tiles start first.
+SA_DEV void tile_coords(int bid, int n_blocks, int n_tiles, int& bh, int& tile) {
+  const int nbh = n_blocks / n_tiles;
+  int logical;
+  if ((nbh & 7) == 0) {
+    const int x = bid & 7, idx = bid >> 3;
+    bh = (idx / n_tiles) * 8 + x;
+    logical = idx % n_tiles;
+  } else {
+    const int per = n_blocks >> 3, rem = n_blocks & 7;
+    const int x = bid & 7, idx = bid >> 3;
+    const int l = x * per + (x < rem ? x : rem) + idx;
+    bh = l / n_tiles;
+    logical = l % n_tiles;
+  }
+  tile = n_tiles - 1 - logical;
 }
 
 // Write four consecutive fp32 values as four elements of T.

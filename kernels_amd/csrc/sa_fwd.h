@@ -28,9 +28,8 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
   const int lane = tid & 63, c = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-  const int bid = xcd_remap(blockIdx.x, gridDim.x);
-  const int qt = bid % p.n_tiles;
-  const int bh = bid / p.n_tiles;
+  int bh, qt;
+  tile_coords(blockIdx.x, gridDim.x, p.n_tiles, bh, qt);
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
 
@@ -257,9 +256,8 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   const int lane = tid & 63, c = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-  const int bid = xcd_remap(blockIdx.x, gridDim.x);
-  const int qt = bid % p.n_tiles;
-  const int bh = bid / p.n_tiles;
+  int bh, qt;
+  tile_coords(blockIdx.x, gridDim.x, p.n_tiles, bh, qt);
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
 
