@@ -252,6 +252,9 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   T* smem = reinterpret_cast<T*>(smem_raw);  // [stage][K|V][TK][D]
 
+#ifdef SA_DBG_TIMING2
+  const long long t_start = __builtin_readcyclecounter();
+#endif
   const int tid = threadIdx.x;
   const int lane = tid & 63, c = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -348,6 +351,9 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
 #define TICK(i) { long long tn = __builtin_readcyclecounter(); tacc[i] += tn - tp; tp = tn; }
 #else
 #define TICK(i)
+#endif
+#ifdef SA_DBG_TIMING2
+  const long long t_loop = __builtin_readcyclecounter();
 #endif
   for (int t = kt0; t < kt1; ++t) {
     // tile t has landed once at most the younger tiles' loads are outstanding
@@ -453,6 +459,16 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   }
 
   // ---- epilogue --------------------------------------------------------------------
+#ifdef SA_DBG_TIMING2
+  {
+    const long long t_end = __builtin_readcyclecounter();
+    if (lse_base && lane < 3) {
+      m_run[0] = lane == 0 ? (float)(t_loop - t_start) : lane == 1 ? (float)(t_end - t_loop) : (float)(kt1 - kt0);
+      l_run[0] = 0.5f;
+    }
+    if (lse_base && lane >= 32 && lane < 35) l_run[0] = 0.5f;
+  }
+#endif
 #ifdef SA_DBG_TIMING
   if (lse_base && lane < 6) {
     long long tv = lane == 0 ? tacc[0] : lane == 1 ? tacc[1] : lane == 2 ? tacc[2] : lane == 3 ? tacc[3] : lane == 4 ? tacc[4] : tacc[5];

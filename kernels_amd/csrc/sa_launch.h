@@ -55,7 +55,11 @@ template <typename T> struct Cfg {
 #else
   static constexpr bool fwd2(int D) { return sizeof(T) == 2 && (D == 64 || D == 128); }
 #endif
+#ifdef SA_FWD_TK16
+  static constexpr int FWD_TK = sizeof(T) == 4 ? 32 : SA_FWD_TK16;
+#else
   static constexpr int FWD_TK = sizeof(T) == 4 ? 32 : 64;        // keys per forward step
+#endif
   static constexpr int DQ_TK = 32;                               // keys per dQ step
   static constexpr int DKDV_TQ = 32;                             // queries per dK/dV step
 };
