@@ -626,20 +626,11 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
     for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
   wait_all_loads();
 
-#ifdef SA_DBG_TIMING
-  long long tacc[6] = {0,0,0,0,0,0}; long long tp = __builtin_readcyclecounter();
-#define TICK(i) { long long tn = __builtin_readcyclecounter(); tacc[i] += tn - tp; tp = tn; }
-#else
-#define TICK(i)
-#endif
   for (int t = qt0; t < qt1; ++t) {
     if (NST == 3 && t + 1 < qt1) wait_loads<LPT>();
     else wait_loads<0>();
-    TICK(0)
     __syncthreads();
-    TICK(1)
     if (t + NST - 1 < qt1) issue_tile(t + NST - 1);
-    TICK(2)
 
     const T* Qt = reinterpret_cast<const T*>(stage_ptr(t));
     const T* Gt = Qt + TILE;
@@ -664,7 +655,6 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
       }
       mma_rows<T, D>(s, Qt, qb * 32, kf, lane);    // S[q][key] = Q K^T
       mma_rows<T, D>(dp, Gt, qb * 32, vf, lane);   // dP[q][key] = dO V^T
-      TICK(3)
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
 #pragma unroll
@@ -684,19 +674,11 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
           dp[0][i] = ok ? dp[0][i] : 0.0f;
         }
       }
-      TICK(4)
       mma_tr<T, D>(dv, Gt, qb, s[0], lane);    // dV^T[d][key] += dO^T P
       mma_tr<T, D>(dk, Qt, qb, dp[0], lane);   // dK^T[d][key] += Q^T dS
-      TICK(5)
     }
   }
 
-#ifdef SA_DBG_TIMING
-  if (lane < 6 && krow < T_) {
-    long long tv = lane == 0 ? tacc[0] : lane == 1 ? tacc[1] : lane == 2 ? tacc[2] : lane == 3 ? tacc[3] : lane == 4 ? tacc[4] : tacc[5];
-    dv[0][0] = (float)tv / (float)(qt1 - qt0);
-  }
-#endif
   if (krow < T_) {
     if (krow >= L) {
 #pragma unroll

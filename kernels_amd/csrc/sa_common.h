@@ -141,13 +141,6 @@ template <typename T> SA_DEV typename Elem<T>::Frag negate(typename Elem<T>::Fra
 // Row of a C fragment that register i of half h holds.
 SA_DEV constexpr int crow(int i, int h) { return 8 * (i >> 2) + 4 * h + (i & 3); }
 
-// Fragment g of row `row` of a row-major LDS tile (contraction along the row).
-template <typename T, int PITCH>
-SA_DEV typename Elem<T>::Frag lds_row_frag(const T* tile, int row, int g, int h) {
-  using Frag = typename Elem<T>::Frag;
-  return *reinterpret_cast<const Frag*>(tile + row * PITCH + (g * 2 + h) * Elem<T>::VEC);
-}
-
 // The compiler's scheduler, left alone, issues each LDS read right before the MFMA that
 // consumes it and so exposes the full LDS latency once per MFMA.  pipeline() forces the
 // shape "fetch group n+1, then multiply group n" with scheduling fences between groups:
@@ -174,70 +167,6 @@ SA_DEV void pipeline(LoadF&& load, UseF&& use) {
   }
   sched_fence();
 }
-
-// Chained form: `first` already holds the fragments of group 0 (the caller fetched them
-// during an earlier phase), and tail() runs in the slot where the last group has nothing left
-// to fetch -- the caller uses it to fetch group 0 of its next phase, so that no phase starts
-// with an exposed LDS latency.
-template <int N, int G, typename F, typename LoadF, typename UseF, typename TailF>
-SA_DEV void pipeline_chained(const F (&first)[G], LoadF&& load, UseF&& use, TailF&& tail) {
-  static_assert(N % G == 0, "items must fill whole groups");
-  constexpr int NG = N / G;
-  F buf[2][G];
-#pragma unroll
-  for (int j = 0; j < G; ++j) buf[0][j] = first[j];
-#pragma unroll
-  for (int grp = 0; grp < NG; ++grp) {
-    sched_fence();
-    if (grp + 1 < NG) {
-#pragma unroll
-      for (int j = 0; j < G; ++j) buf[(grp + 1) & 1][j] = load((grp + 1) * G + j);
-    } else {
-      tail();
-    }
-#pragma unroll
-    for (int j = 0; j < G; ++j) use(grp * G + j, buf[grp & 1][j]);
-  }
-  sched_fence();
-}
-
-// Per-lane address helpers for the two fragment kinds, for callers that drive pipeline*()
-// themselves.  RowFrags: fragment g of row (row0 + c) of a row-major tile.  TrFrags: the
-// transposed fragment (half, m) of 32-row block rb, as two 4-row runs 8 rows apart.
-template <typename T, int D> struct RowFrags {
-  using G_ = TileGeom<T, D>;
-  using Frag = typename Elem<T>::Frag;
-  int lane_off;   // element offset of this lane's row start inside a 32-row block
-  int sw, h;
-  SA_DEV void init(int lane) {
-    const int c = lane & 31;
-    h = lane >> 5;
-    lane_off = c * G_::PITCH;
-    sw = G_::swz(c);
-  }
-  SA_DEV Frag load(const T* tile, int row0, int g) const {
-    return *reinterpret_cast<const Frag*>(tile + row0 * G_::PITCH + lane_off + (((g * 2 + h) ^ sw) * Elem<T>::VEC));
-  }
-};
-
-template <typename T, int D> struct TrFrags {
-  using G_ = TileGeom<T, D>;
-  using Frag = typename Elem<T>::Frag;
-  int r_lo, col;
-  SA_DEV void init(int lane) {
-    const int g16 = lane >> 4, j = lane & 15;
-    r_lo = 4 * (g16 >> 1) + (j >> 2);
-    col = (g16 & 1) * 16 + 4 * (j & 3);
-  }
-  SA_DEV Frag load(const T* tile, int rb, int half, int m) const {
-    const T* blk = tile + rb * 32 * G_::PITCH;
-    const T* p0 = blk + G_::off(half * 16 + r_lo, m * 32 + col);
-    const T* p1 = blk + G_::off(half * 16 + 8 + r_lo, m * 32 + col);
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p0));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p1));
-    return __builtin_bit_cast(Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-  }
-};
 
 // acc[nb] += A_nb * B for NB row blocks of a row-major LDS tile that share the register
 // fragments bf:  acc[nb][row r][col c] += sum_k tile[row0 + nb*32 + r][k] * B[k][c].
@@ -481,21 +410,8 @@ SA_DEV void tile_coords(int bid, int n_blocks, int n_tiles, int& bh, int& tile) 
   int logical;
   if ((nbh & 7) == 0) {
     const int x = bid & 7, idx = bid >> 3;
-#if defined(SA_MAP_TILE_MAJOR)
-    const int nl = nbh >> 3;                       // (batch, head) pairs per XCD
-    bh = (idx % nl) * 8 + x;
-    logical = idx / nl;
-#elif defined(SA_MAP_GROUP4)
-    // groups of 4 consecutive tiles of one pair, pairs interleaved
-    const int nl = nbh >> 3;
-    const int grp = idx / (4 * nl), within = idx % (4 * nl);
-    bh = (within / 4) * 8 + x;
-    logical = grp * 4 + (within % 4);
-    if (logical >= n_tiles) { bh = -1; }
-#else
     bh = (idx / n_tiles) * 8 + x;
     logical = idx % n_tiles;
-#endif
   } else {
     const int per = n_blocks >> 3, rem = n_blocks & 7;
     const int x = bid & 7, idx = bid >> 3;

@@ -101,12 +101,6 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
   wait_all_loads();
   __syncthreads();
 
-#ifdef SA_DBG_TIMING
-  long long tacc[6] = {0,0,0,0,0,0}; long long tp = __builtin_readcyclecounter();
-#define TICK(i) { long long tn = __builtin_readcyclecounter(); tacc[i] += tn - tp; tp = tn; }
-#else
-#define TICK(i)
-#endif
   for (int t = kt0; t < kt1; ++t) {
     const int cur = (t - kt0) & 1;
     const T* Kt = smem + cur * 2 * TILE;
@@ -117,7 +111,6 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
       sv.load(vbase, p.v_st, (t + 1) * TK, T_ - 1, tid);
     }
     const int k0 = t * TK;
-    TICK(0)
 
     // S^T[key][q] = K Q^T
     f32x16 s[KBN];
@@ -127,7 +120,6 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
       for (int i = 0; i < 16; ++i) s[kb][i] = 0.0f;
     mma_rows<T, D>(s, Kt, 0, qf, lane);
 
-    TICK(1)
     // Online softmax in base 2 on the raw scores: p = exp2(s*sl2e - m).  The two halves of
     // the wave hold disjoint keys of the same query, so only the max crosses lanes inside
     // the loop.  The reference point m moves only when the tile's max exceeds it by more
@@ -188,31 +180,19 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
       for (int i = 0; i < 16; ++i) rs += s[kb][i];
     l_run += rs;
 
-    TICK(2)
     // O^T[d][q] += V^T P^T
 #pragma unroll
     for (int kb = 0; kb < KBN; ++kb) mma_tr<T, D>(oacc, Vt, kb, s[kb], lane);
 
-    TICK(3)
     if (more) {
       T* nxt = smem + (cur ^ 1) * 2 * TILE;
       sk.store(nxt, tid);
       sv.store(nxt + TILE, tid);
     }
-    TICK(4)
     __syncthreads();
-    TICK(5)
   }
 
   // ---- epilogue --------------------------------------------------------------------
-#ifdef SA_DBG_TIMING
-  if (lse_base && lane < 6) {
-    long long tv = lane == 0 ? tacc[0] : lane == 1 ? tacc[1] : lane == 2 ? tacc[2] : lane == 3 ? tacc[3] : lane == 4 ? tacc[4] : tacc[5];
-    m_run = (float)tv / (float)(kt1 - kt0);
-    l_run = 0.5f;
-  }
-  if (lse_base && lane >= 32 && lane < 38) l_run = 0.5f;
-#endif
   const float l_tot = half_sum(l_run);
   const bool valid = qrow < L;
   if (qrow < T_) {
@@ -252,9 +232,6 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
   T* smem = reinterpret_cast<T*>(smem_raw);  // [stage][K|V][TK][D]
 
-#ifdef SA_DBG_TIMING2
-  const long long t_start = __builtin_readcyclecounter();
-#endif
   const int tid = threadIdx.x;
   const int lane = tid & 63, c = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -345,31 +322,16 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   }
   wait_all_loads();   // Q fragments (and, as loads complete in order, the first tiles)
 
-#undef TICK
-#ifdef SA_DBG_TIMING
-  long long tacc[6] = {0,0,0,0,0,0}; long long tp = __builtin_readcyclecounter();
-#define TICK(i) { long long tn = __builtin_readcyclecounter(); tacc[i] += tn - tp; tp = tn; }
-#else
-#define TICK(i)
-#endif
-#ifdef SA_DBG_TIMING2
-  const long long t_loop = __builtin_readcyclecounter();
-#endif
   for (int t = kt0; t < kt1; ++t) {
     // tile t has landed once at most the younger tiles' loads are outstanding
     if (NST == 3 && t + 1 < kt1) wait_loads<LPT>();
     else wait_loads<0>();
-    TICK(0)
     __syncthreads();   // every wave's share is visible; stage (t-1) % NST is free again
-    TICK(1)
-#ifndef SA_DBG_NOLOAD
     if (t + NST - 1 < kt1) issue_tile(t + NST - 1);
-#endif
 
     const T* Kt = smem + ((t - kt0) % NST) * STAGE;
     const T* Vt = Kt + TILE;
     const int k0 = t * TK;
-    TICK(5)
 
     // S^T[key][q] = K Q^T for the QB query blocks
     f32x16 s[QB][KBN];
@@ -379,14 +341,10 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
       for (int kb = 0; kb < KBN; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[qb][kb][i] = 0.0f;
-#ifndef SA_DBG_NOQK
     mma_rows_n<T, D>(s, Kt, 0, qf, lane);
-#endif
 
-    TICK(2)
     const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
     Frag pb[QB][KBN][2];
-#ifndef SA_DBG_NOSOFTMAX
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       float mx = -INFINITY;
@@ -439,43 +397,17 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
       l_run[qb] += rs;
     }
 
-#else
-    for (int qb = 0; qb < QB; ++qb) for (int kb = 0; kb < KBN; ++kb) pack_c<T>(pb[qb][kb], s[qb][kb]);
-#endif
-    TICK(3)
     // O^T[d][q] += V^T P^T
 #pragma unroll
     for (int kb = 0; kb < KBN; ++kb) {
       Frag bq[QB][2];
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) bq[qb][0] = pb[qb][kb][0], bq[qb][1] = pb[qb][kb][1];
-#ifndef SA_DBG_NOPV
       mma_tr_n<T, D>(oacc, Vt, kb, bq, lane);
-      TICK(4)
-#else
-      for (int qb = 0; qb < QB; ++qb) for (int e = 0; e < 8; ++e) oacc[qb][0][e] += (float)bq[qb][0][e] + (float)bq[qb][1][e];
-#endif
     }
   }
 
   // ---- epilogue --------------------------------------------------------------------
-#ifdef SA_DBG_TIMING2
-  {
-    const long long t_end = __builtin_readcyclecounter();
-    if (lse_base && lane < 3) {
-      m_run[0] = lane == 0 ? (float)(t_loop - t_start) : lane == 1 ? (float)(t_end - t_loop) : (float)(kt1 - kt0);
-      l_run[0] = 0.5f;
-    }
-    if (lse_base && lane >= 32 && lane < 35) l_run[0] = 0.5f;
-  }
-#endif
-#ifdef SA_DBG_TIMING
-  if (lse_base && lane < 6) {
-    long long tv = lane == 0 ? tacc[0] : lane == 1 ? tacc[1] : lane == 2 ? tacc[2] : lane == 3 ? tacc[3] : lane == 4 ? tacc[4] : tacc[5];
-    m_run[0] = (float)tv / (float)(kt1 - kt0);
-    l_run[0] = 0.5f;
-  }
-#endif
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const float l_tot = half_sum(l_run[qb]);
