@@ -488,8 +488,7 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
       f32x16 s[1], dp[1];
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[0][i] = 0.0f, dp[0][i] = 0.0f;
-      mma_rows<T, D>(s, Kt, kb * 32, qf, lane);
-      mma_rows<T, D>(dp, Vt, kb * 32, gf, lane);
+      mma_rows_pair<T, D>(s[0], dp[0], Kt, Vt, kb * 32, qf, gf, lane);
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const float pr = fast_exp2(__builtin_fmaf(s[0][i], sl2e, -lse_q));
@@ -653,8 +652,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
         l4[g4] = *reinterpret_cast<const f32x4*>(chunk);
         d4[g4] = *reinterpret_cast<const f32x4*>(chunk + RPW);
       }
-      mma_rows<T, D>(s, Qt, qb * 32, kf, lane);    // S[q][key] = Q K^T
-      mma_rows<T, D>(dp, Gt, qb * 32, vf, lane);   // dP[q][key] = dO V^T
+      // S[q][key] = Q K^T and dP[q][key] = dO V^T
+      mma_rows_pair<T, D>(s[0], dp[0], Qt, Gt, qb * 32, kf, vf, lane);
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
 #pragma unroll
@@ -674,8 +673,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
           dp[0][i] = ok ? dp[0][i] : 0.0f;
         }
       }
-      mma_tr<T, D>(dv, Gt, qb, s[0], lane);    // dV^T[d][key] += dO^T P
-      mma_tr<T, D>(dk, Qt, qb, dp[0], lane);   // dK^T[d][key] += Q^T dS
+      // dV^T[d][key] += dO^T P and dK^T[d][key] += Q^T dS
+      mma_tr_pair<T, D>(dv, dk, Gt, Qt, qb, s[0], dp[0], lane);
     }
   }
 

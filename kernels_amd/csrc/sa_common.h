@@ -271,6 +271,66 @@ template <typename T> SA_DEV void pack_c(typename Elem<T>::Frag (&b)[2], const f
     for (int e = 0; e < 8; ++e) b[half][e] = (T)P[half * 8 + e];
 }
 
+// Two products that share the pipeline: acc0 += A0 * B0 and acc1 += A1 * B1, where A0 and A1
+// are the same 32 rows of two row-major LDS tiles (scores from Q and K, dP from dO and V).
+// One fragment stream means one exposed LDS latency instead of two.
+template <typename T, int D, int NF>
+SA_DEV void mma_rows_pair(f32x16& acc0, f32x16& acc1, const T* tile0, const T* tile1, int row0,
+                          const typename Elem<T>::Frag (&b0)[NF], const typename Elem<T>::Frag (&b1)[NF],
+                          int lane) {
+  using G_ = TileGeom<T, D>;
+  using Frag = typename Elem<T>::Frag;
+  static_assert(NF == G_::NF, "one register fragment per 2*VEC slice of the head dimension");
+  constexpr int PITCH = G_::PITCH, VEC = Elem<T>::VEC;
+  const int c = lane & 31, h = lane >> 5;
+  constexpr int N = 2 * NF, G = N < 4 ? N : 4;
+  const int off = (row0 + c) * PITCH;
+  const int sw = G_::swz(c);
+  pipeline<N, G>(
+      [&](int it) {
+        const T* base = (it < NF ? tile0 : tile1) + off;
+        return *reinterpret_cast<const Frag*>(base + ((((it % NF) * 2 + h) ^ sw) * VEC));
+      },
+      [&](int it, const Frag& a) {
+        if (it < NF) mma(acc0, a, b0[it]);
+        else mma(acc1, a, b1[it - NF]);
+      });
+}
+
+// Likewise for the transposed products: acc0[m] += X0^T * P0 and acc1[m] += X1^T * P1 over the
+// same 32-row block of two tiles (dV from dO and P, dK from Q and dS).  16-bit types only.
+template <typename T, int D, int NM>
+SA_DEV void mma_tr_pair(f32x16 (&acc0)[NM], f32x16 (&acc1)[NM], const T* X0, const T* X1, int rb,
+                        const f32x16& P0, const f32x16& P1, int lane) {
+  using E = Elem<T>;
+  using G_ = TileGeom<T, D>;
+  using Frag = typename E::Frag;
+  static_assert(E::HALF && NM == G_::DB, "transposing reads exist for 16-bit elements only");
+  constexpr int PITCH = G_::PITCH;
+  const int g16 = lane >> 4, j = lane & 15;
+  const int r_lo = 4 * (g16 >> 1) + (j >> 2);
+  const int col = (g16 & 1) * 16 + 4 * (j & 3);
+  Frag b0[2], b1[2];
+  pack_c<T>(b0, P0);
+  pack_c<T>(b1, P1);
+  constexpr int N = 4 * NM, G = N < 4 ? N : 4;
+  pipeline<N, G>(
+      [&](int it) {
+        const int k2 = it % (2 * NM), half = k2 / NM, m = k2 % NM;
+        const T* blk = (it < 2 * NM ? X0 : X1) + rb * 32 * PITCH;
+        const T* p0 = blk + G_::off(half * 16 + r_lo, m * 32 + col);
+        const T* p1 = blk + G_::off(half * 16 + 8 + r_lo, m * 32 + col);
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p0));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p1));
+        return __builtin_bit_cast(Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      },
+      [&](int it, const Frag& a) {
+        const int k2 = it % (2 * NM), half = k2 / NM, m = k2 % NM;
+        if (it < 2 * NM) mma(acc0[m], a, b0[half]);
+        else mma(acc1[m], a, b1[half]);
+      });
+}
+
 // 16-bit only: acc[q][m] += X^T * B[q] for 32-row block rb of tile X, B[q] packed by pack_c.
 template <typename T, int D, int NQ, int NM>
 SA_DEV void mma_tr_n(f32x16 (&acc)[NQ][NM], const T* X, int rb, const typename Elem<T>::Frag (&b)[NQ][2],
