@@ -158,6 +158,14 @@ def cpu_baseline(max_seconds=20.0):
     }
 
 
+# HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (separate --pmc runs of this script, scaled by
+# what the same counters read for the 1 GiB copy of --calibrate-copy: x2.000 and x1.000).  Counter runs
+# cannot be made from inside a timed run, so the figures of the committed profile summary are quoted here.
+HBM_BYTES_PER_LAUNCH = {
+    "headline_bf16_T16384_D128": {"fwd": 1.603e9, "delta": 5.411e8, "dq": 2.033e9, "dkdv": 1.731e9},
+}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -228,7 +236,8 @@ def main():
         "kernel_tflops": {n: kernel_flops[n] / (kt[n] * 1e-3) / 1e12 for n in kernel_flops},
         "delta_gbs": (2.0 * N * D * es + 4.0 * N) / (kt["delta"] * 1e-3) / 1e9,
         "roofline": {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None},
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
+                     "traffic": HBM_BYTES_PER_LAUNCH.get(args.workload, {}).get(dom)},
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
