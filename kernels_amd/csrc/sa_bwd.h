@@ -459,11 +459,16 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
     for (int g = 0; g < NF; ++g) {
       qf[g] = *reinterpret_cast<const Frag*>(qp + (g * 2 + h) * E::VEC);
       if (neg) qf[g] = negate<T>(qf[g]);
-      gf[g] = *reinterpret_cast<const Frag*>(gp + (g * 2 + h) * E::VEC);
+      // dO enters negated: the dP accumulator starts at delta and ends at delta - dP, which
+      // saves the subtraction per element; the sign is put back by the scale of the store
+      gf[g] = negate<T>(*reinterpret_cast<const Frag*>(gp + (g * 2 + h) * E::VEC));
     }
     lse_q = qrow < L ? p.lse[(int64_t)bh * T_ + qr] : INFINITY;   // rows past L: P = exp2(-inf) = 0
     delta_q = p.delta[(int64_t)bh * T_ + qr];
   }
+  f32x16 dinit;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) dinit[i] = delta_q;
 
   f32x16 acc[DB];
 #pragma unroll
@@ -487,12 +492,13 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
     for (int kb = 0; kb < KBN; ++kb) {
       f32x16 s[1], dp[1];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[0][i] = 0.0f, dp[0][i] = 0.0f;
+      for (int i = 0; i < 16; ++i) s[0][i] = 0.0f;
+      dp[0] = dinit;
       mma_rows_pair<T, D>(s[0], dp[0], Kt, Vt, kb * 32, qf, gf, lane);
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const float pr = fast_exp2(__builtin_fmaf(s[0][i], sl2e, -lse_q));
-        s[0][i] = pr * (dp[0][i] - delta_q);
+        s[0][i] = pr * dp[0][i];   // = -dS
       }
       if (!interior) {
 #pragma unroll
@@ -501,7 +507,7 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
           s[0][i] = (key < lo || key >= hi) ? 0.0f : s[0][i];
         }
       }
-      mma_tr<T, D>(acc, Kt, kb, s[0], lane);   // dQ^T[d][q] += K^T dS^T
+      mma_tr<T, D>(acc, Kt, kb, s[0], lane);   // -dQ^T[d][q] += K^T (-dS^T)
     }
   }
 
@@ -512,7 +518,7 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
     }
-    store_acc_T<T, D, DB>(dq_base + (int64_t)qrow * D, acc, p.scale, h);
+    store_acc_T<T, D, DB>(dq_base + (int64_t)qrow * D, acc, -p.scale, h);
   }
 }
 
@@ -614,7 +620,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
     for (int g = 0; g < NF; ++g) {
       kf[g] = *reinterpret_cast<const Frag*>(kp + (g * 2 + h) * E::VEC);
       if (neg) kf[g] = negate<T>(kf[g]);
-      vf[g] = *reinterpret_cast<const Frag*>(vp + (g * 2 + h) * E::VEC);
+      // V enters negated: the dP accumulator starts at delta and ends at delta - dP
+      vf[g] = negate<T>(*reinterpret_cast<const Frag*>(vp + (g * 2 + h) * E::VEC));
     }
   }
 
@@ -641,16 +648,18 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
     for (int qb = 0; qb < QBN; ++qb) {
       f32x16 s[1], dp[1];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[0][i] = 0.0f, dp[0][i] = 0.0f;
-      // lse / delta of the 16 rows this lane holds: fetched ahead of the products so that
-      // their LDS latency is not exposed in the element-wise phase
-      f32x4 l4[4], d4[4];
+      for (int i = 0; i < 16; ++i) s[0][i] = 0.0f;
+      // lse / delta of the 16 rows this lane holds, fetched ahead of the products; delta is
+      // read straight into the dP accumulator
+      f32x4 l4[4];
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         const int r = qb * 32 + 8 * g4 + 4 * h;     // tile row of 4 consecutive C-fragment rows
         const float* chunk = ld_t + (r / RPW) * 2 * RPW + (r % RPW);
         l4[g4] = *reinterpret_cast<const f32x4*>(chunk);
-        d4[g4] = *reinterpret_cast<const f32x4*>(chunk + RPW);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(chunk + RPW);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dp[0][4 * g4 + e] = d4[e];
       }
       // S[q][key] = Q K^T and dP[q][key] = dO V^T
       mma_rows_pair<T, D>(s[0], dp[0], Qt, Gt, qb * 32, kf, vf, lane);
@@ -661,7 +670,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
           const int i = 4 * g4 + e;
           const float pr = fast_exp2(__builtin_fmaf(s[0][i], sl2e, -l4[g4][e]));
           s[0][i] = pr;
-          dp[0][i] = pr * (dp[0][i] - d4[g4][e]);
+          dp[0][i] = pr * dp[0][i];   // = -dS
         }
       }
       if (!interior) {
@@ -673,7 +682,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
           dp[0][i] = ok ? dp[0][i] : 0.0f;
         }
       }
-      // dV^T[d][key] += dO^T P and dK^T[d][key] += Q^T dS
+      // dV^T[d][key] += dO^T P and -dK^T[d][key] += Q^T (-dS)
       mma_tr_pair<T, D>(dv, dk, Gt, Qt, qb, s[0], dp[0], lane);
     }
   }
@@ -685,7 +694,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
     }
-    store_acc_T<T, D, DB>(dk_base + (int64_t)krow * D, dk, p.scale, h);
+    store_acc_T<T, D, DB>(dk_base + (int64_t)krow * D, dk, -p.scale, h);
     store_acc_T<T, D, DB>(dv_base + (int64_t)krow * D, dv, 1.0f, h);
   }
 }

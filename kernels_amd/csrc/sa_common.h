@@ -132,6 +132,34 @@ SA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 // that fmaxf() costs per operand.
 SA_DEV float fast_max(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, INFINITY); }
 
+// max(a, b, c) in one instruction.  Written as asm because the three-operand form is only
+// selected from fmaxf() chains together with a canonicalising move per operand.
+SA_DEV float fast_max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+// acc + the sum of the eight 16-bit values of a fragment: four dot products with (1, 1), i.e.
+// half a vector instruction per element, and the sum is over the rounded values that the
+// following matrix product consumes.
+SA_DEV float sum_frag(bf16x8 f, float acc) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{f[2 * j], f[2 * j + 1]}, one, acc, false);
+  return acc;
+}
+SA_DEV float sum_frag(f16x8 f, float acc) {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    acc = __builtin_amdgcn_fdot2(f16x2{f[2 * j], f[2 * j + 1]}, one, acc, false);
+  return acc;
+}
+
 template <typename T> SA_DEV typename Elem<T>::Frag negate(typename Elem<T>::Frag f) {
   u32x4 u = __builtin_bit_cast(u32x4, f);
   u ^= Elem<T>::SIGN;

@@ -349,10 +349,15 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
     for (int qb = 0; qb < QB; ++qb) {
       float mx = -INFINITY;
       if (interior) {
+        float mk[KBN];   // one chain per key block, so that consecutive instructions are independent
 #pragma unroll
-        for (int kb = 0; kb < KBN; ++kb)
+        for (int kb = 0; kb < KBN; ++kb) mk[kb] = -INFINITY;
 #pragma unroll
-          for (int i = 0; i < 16; ++i) mx = fast_max(mx, s[qb][kb][i]);
+        for (int i = 0; i < 16; i += 2)
+#pragma unroll
+          for (int kb = 0; kb < KBN; ++kb) mk[kb] = fast_max3(mk[kb], s[qb][kb][i], s[qb][kb][i + 1]);
+#pragma unroll
+        for (int kb = 0; kb < KBN; ++kb) mx = fast_max(mx, mk[kb]);
       } else {
 #pragma unroll
         for (int kb = 0; kb < KBN; ++kb)
@@ -387,14 +392,14 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
             s[qb][kb][i] = (key >= lo[qb] && key < hi[qb]) ? s[qb][kb][i] : 0.0f;
           }
       }
-      float rs = 0.0f;
+      float rs[2] = {0.0f, 0.0f};
 #pragma unroll
       for (int kb = 0; kb < KBN; ++kb) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) rs += s[qb][kb][i];
         pack_c<T>(pb[qb][kb], s[qb][kb]);
+        rs[0] = sum_frag(pb[qb][kb][0], rs[0]);
+        rs[1] = sum_frag(pb[qb][kb][1], rs[1]);
       }
-      l_run[qb] += rs;
+      l_run[qb] += rs[0] + rs[1];
     }
 
     // O^T[d][q] += V^T P^T
