@@ -423,6 +423,10 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
   const int wq_last = q0 + wave * 32 + 31 < L ? q0 + wave * 32 + 31 : L - 1;
   const int hi_min = (wq_first / C + 1) * C < L ? (wq_first / C + 1) * C : L;
   const int lo_max = (wq_last / C > R ? wq_last / C - R : 0) * C;
+  // keys any query of this wave can see; a wave whose queries are all padding sees none
+  const bool wave_live = q0 + wave * 32 < L;
+  const int lo_min = (wq_first / C > R ? wq_first / C - R : 0) * C;
+  const int hi_max = !wave_live ? 0 : ((wq_last / C + 1) * C < L ? (wq_last / C + 1) * C : L);
   const int gq_last = q0 + TQ - 1 < L ? q0 + TQ - 1 : L - 1;
   const int lo_wg = (q0 / C > R ? q0 / C - R : 0) * C;
   const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
@@ -486,6 +490,7 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
     const T* Kt = smem + ((t - kt0) % NST) * STAGE;
     const T* Vt = Kt + TILE;
     const int k0 = t * TK;
+    if (k0 + TK <= lo_min || k0 >= hi_max) continue;   // outside this wave's windows
     const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
 
 #pragma unroll
@@ -575,6 +580,9 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
   const int wk_first = k0 + wave * 32 < L ? k0 + wave * 32 : L - 1;
   const int wk_last = k0 + wave * 32 + 31 < L ? k0 + wave * 32 + 31 : L - 1;
   const int qhi_min = win_hi(wk_first), qlo_max = win_lo(wk_last);
+  // queries that can see any key of this wave; a wave whose keys are all padding has none
+  const bool wave_live = k0 + wave * 32 < L;
+  const int qlo_min = win_lo(wk_first), qhi_max = wave_live ? win_hi(wk_last) : 0;
   const int gk_last = k0 + TKB - 1 < L ? k0 + TKB - 1 : L - 1;
   const int qt0 = win_lo(k0) / TQ, qt1 = (win_hi(gk_last) + TQ - 1) / TQ;
 
@@ -642,6 +650,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
     const T* Gt = Qt + TILE;
     const float* ld_t = reinterpret_cast<const float*>(stage_ptr(t) + 2 * TILE * sizeof(T));
     const int qs = t * TQ;
+    if (qs + TQ <= qlo_min || qs >= qhi_max) continue;   // outside this wave's windows
     const bool interior = (qs >= qlo_max) && (qs + TQ <= qhi_min);
 
 #pragma unroll

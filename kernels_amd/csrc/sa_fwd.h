@@ -271,6 +271,10 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   const int wq_last = q0 + wave * WQ + WQ - 1 < L ? q0 + wave * WQ + WQ - 1 : L - 1;
   const int hi_min = (wq_first / C + 1) * C < L ? (wq_first / C + 1) * C : L;
   const int lo_max = (wq_last / C > R ? wq_last / C - R : 0) * C;
+  // keys any query of this wave can see; a wave whose queries are all padding sees none
+  const bool wave_live = q0 + wave * WQ < L;
+  const int lo_min = (wq_first / C > R ? wq_first / C - R : 0) * C;
+  const int hi_max = !wave_live ? 0 : ((wq_last / C + 1) * C < L ? (wq_last / C + 1) * C : L);
   const int gq_last = q0 + TQ - 1 < L ? q0 + TQ - 1 : L - 1;
   const int lo_wg = (q0 / C > R ? q0 / C - R : 0) * C;
   const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
@@ -332,6 +336,8 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
     const T* Kt = smem + ((t - kt0) % NST) * STAGE;
     const T* Vt = Kt + TILE;
     const int k0 = t * TK;
+    // the workgroup's key range is the union over its waves; skip what this wave cannot see
+    if (k0 + TK <= lo_min || k0 >= hi_max) continue;
 
     // S^T[key][q] = K Q^T for the QB query blocks
     f32x16 s[QB][KBN];

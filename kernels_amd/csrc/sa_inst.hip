@@ -54,19 +54,23 @@ static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 #endif
 
 #if SA_KIND == 0
+template <int D, int NW> static int fwd2_launch(FwdParams p, hipStream_t st) {
+  using C = Cfg<ElemT>;
+  constexpr int TQ = NW * C::FWD2_QB * 32;
+  constexpr size_t lds = (size_t)C::FWD2_NST * 2 * C::FWD_TK * D * sizeof(ElemT);
+  auto kern = fwd2_kernel<ElemT, D, C::FWD2_QB, NW, C::FWD_TK, C::FWD2_NST>;
+  static std::once_flag once;
+  if (int rc = prepare(kern, lds, once)) return rc;
+  p.n_tiles = (int)ceil_div(p.T, TQ);
+  const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+  if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), lds, st, p);
+  return (int)hipGetLastError();
+}
 template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
-    constexpr int TQ = C::FWD2_NW * C::FWD2_QB * 32;
-    constexpr size_t lds = (size_t)C::FWD2_NST * 2 * C::FWD_TK * D * sizeof(ElemT);
-    auto kern = fwd2_kernel<ElemT, D, C::FWD2_QB, C::FWD2_NW, C::FWD_TK, C::FWD2_NST>;
-    static std::once_flag once;
-    if (int rc = prepare(kern, lds, once)) return rc;
-    p.n_tiles = (int)ceil_div(p.T, TQ);
-    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
-    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::FWD2_NW * 64), lds, st, p);
-    return (int)hipGetLastError();
+    return C::wide(p.C) ? fwd2_launch<D, C::WIDE_NW>(p, st) : fwd2_launch<D, C::NARROW_NW>(p, st);
   } else {
     constexpr int TQ = C::NW * 32;
     constexpr size_t lds = (size_t)2 * 2 * C::FWD_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
@@ -99,19 +103,23 @@ template <> int launch_delta<ElemT, SA_DGROUP>(const DeltaParams& p, int D, hipS
   SA_FOR_EACH_D(X)
 #undef X
 }
+template <int D, int NW> static int dq2_launch(BwdParams p, hipStream_t st) {
+  using C = Cfg<ElemT>;
+  constexpr int TQ = NW * 32;
+  constexpr size_t lds = (size_t)C::DQ2_NST * 2 * C::DQ2_TK * D * sizeof(ElemT);
+  auto kern = dq2_kernel<ElemT, D, NW, C::DQ2_TK, C::DQ2_NST>;
+  static std::once_flag once;
+  if (int rc = prepare(kern, lds, once)) return rc;
+  p.n_tiles = (int)ceil_div(p.T, TQ);
+  const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+  if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), lds, st, p);
+  return (int)hipGetLastError();
+}
 template <int D> static int dq_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
-    constexpr int TQ = C::DQ2_NW * 32;
-    constexpr size_t lds = (size_t)C::DQ2_NST * 2 * C::DQ2_TK * D * sizeof(ElemT);
-    auto kern = dq2_kernel<ElemT, D, C::DQ2_NW, C::DQ2_TK, C::DQ2_NST>;
-    static std::once_flag once;
-    if (int rc = prepare(kern, lds, once)) return rc;
-    p.n_tiles = (int)ceil_div(p.T, TQ);
-    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
-    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::DQ2_NW * 64), lds, st, p);
-    return (int)hipGetLastError();
+    return C::wide(p.C) ? dq2_launch<D, C::WIDE_NW>(p, st) : dq2_launch<D, C::NARROW_NW>(p, st);
   } else {
     constexpr int TQ = C::NW * 32;
     constexpr size_t lds = (size_t)2 * 2 * C::DQ_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);

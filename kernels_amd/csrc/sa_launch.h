@@ -18,9 +18,6 @@ template <typename T, int DGROUP> int launch_dkdv(const BwdParams& p, int D, hip
 #ifndef SA_FWD2_QB
 #define SA_FWD2_QB 1
 #endif
-#ifndef SA_DQ2_NW
-#define SA_DQ2_NW 8
-#endif
 #ifndef SA_DQ2_TK
 #define SA_DQ2_TK 64
 #endif
@@ -36,17 +33,19 @@ template <typename T, int DGROUP> int launch_dkdv(const BwdParams& p, int D, hip
 #ifndef SA_DKDV2_NST
 #define SA_DKDV2_NST 2
 #endif
-#ifndef SA_FWD2_NW
-#define SA_FWD2_NW 8
-#endif
 #ifndef SA_FWD2_NST
 #define SA_FWD2_NST 2
 #endif
 template <typename T> struct Cfg {
   static constexpr int NW = 4;                                   // waves per workgroup
   // 16-bit, D in {64, 128}: forward kernel with QB query blocks per wave and NST LDS stages
-  static constexpr int FWD2_NW = SA_FWD2_NW;
-  static constexpr int DQ2_NW = SA_DQ2_NW, DQ2_TK = SA_DQ2_TK, DQ2_NST = SA_DQ2_NST;
+  // The forward and dQ kernels come in two widths, chosen per call from the chunk size:
+  // 8 waves (256 queries) share each key tile among more waves, which pays once the
+  // workgroup's queries lie in one chunk; with smaller chunks the union of the waves'
+  // windows grows and 4 waves (128 queries) waste less of every tile.
+  static constexpr int WIDE_NW = 8, NARROW_NW = 4;
+  static constexpr bool wide(int chunk) { return chunk >= 256; }
+  static constexpr int DQ2_TK = SA_DQ2_TK, DQ2_NST = SA_DQ2_NST;
   static constexpr int DKDV2_NW = SA_DKDV2_NW, DKDV2_TQ = SA_DKDV2_TQ, DKDV2_NST = SA_DKDV2_NST;
   static constexpr int FWD2_QB = SA_FWD2_QB;
   static constexpr int FWD2_NST = SA_FWD2_NST;
