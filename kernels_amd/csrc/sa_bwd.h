@@ -506,11 +506,9 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
         s[0][i] = pr * dp[0][i];   // = -dS
       }
       if (!interior) {
+        const uint32_t rm = row_mask(lo - (k0 + kb * 32), hi - (k0 + kb * 32), h);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = k0 + kb * 32 + crow(i, h);
-          s[0][i] = (key < lo || key >= hi) ? 0.0f : s[0][i];
-        }
+        for (int i = 0; i < 16; ++i) s[0][i] = keep_or_zero(s[0][i], keep_bits(rm, i));
       }
       mma_tr<T, D>(acc, Kt, kb, s[0], lane);   // -dQ^T[d][q] += K^T (-dS^T)
     }
@@ -683,12 +681,12 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
         }
       }
       if (!interior) {
+        const uint32_t rm = row_mask(qlo - (qs + qb * 32), qhi - (qs + qb * 32), h);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const int qr = qs + qb * 32 + crow(i, h);
-          const bool ok = qr >= qlo && qr < qhi;
-          s[0][i] = ok ? s[0][i] : 0.0f;
-          dp[0][i] = ok ? dp[0][i] : 0.0f;
+          const uint32_t keep = keep_bits(rm, i);
+          s[0][i] = keep_or_zero(s[0][i], keep);
+          dp[0][i] = keep_or_zero(dp[0][i], keep);
         }
       }
       // dV^T[d][key] += dO^T P and -dK^T[d][key] += Q^T (-dS)

@@ -160,6 +160,26 @@ SA_DEV float sum_frag(f16x8 f, float acc) {
   return acc;
 }
 
+// Masks for the edge of a window.  Rows [a, b) of a 32-row block are allowed; row_mask() packs
+// that into one bit per row, pre-shifted for the lane's half so that the bit of accumulator
+// register i sits at the compile-time position 8*(i/4) + i%4.  keep_bits() expands one bit
+// into all-ones / zero; an element is then kept or cleared with a single bitwise operation
+// instead of two compares, a mask merge and a select.
+SA_DEV uint32_t row_mask(int a, int b, int h) {
+  a = a < 0 ? 0 : a;
+  b = b < 0 ? 0 : b;
+  const uint32_t below_b = b >= 32 ? 0xFFFFFFFFu : ((1u << b) - 1u);
+  const uint32_t below_a = a >= 32 ? 0xFFFFFFFFu : ((1u << a) - 1u);
+  return (below_b & ~below_a) >> (4 * h);
+}
+SA_DEV uint32_t keep_bits(uint32_t m, int i) {
+  return (uint32_t)__builtin_amdgcn_sbfe((int)m, 8 * (i >> 2) + (i & 3), 1);
+}
+SA_DEV float keep_or_zero(float x, uint32_t keep) { return __uint_as_float(__float_as_uint(x) & keep); }
+SA_DEV float keep_or_neg_inf(float x, uint32_t keep) {
+  return __uint_as_float((__float_as_uint(x) & keep) | (0xFF800000u & ~keep));
+}
+
 template <typename T> SA_DEV typename Elem<T>::Frag negate(typename Elem<T>::Frag f) {
   u32x4 u = __builtin_bit_cast(u32x4, f);
   u ^= Elem<T>::SIGN;

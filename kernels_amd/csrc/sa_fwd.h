@@ -280,7 +280,8 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
   const int kt0 = lo_wg / TK, kt1 = (hi_wg + TK - 1) / TK;
 
-  const float sl2e = fabsf(p.scale_log2e);
+  // never exactly 0, so that a masked score of -inf stays -inf after scaling
+  const float sl2e = fmaxf(fabsf(p.scale_log2e), 1e-30f);
   const bool neg = p.scale_log2e < 0.0f;
 
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh;
@@ -353,8 +354,17 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
     Frag pb[QB][KBN][2];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
+      if (!interior) {
+        // keys outside [lo, hi) score -inf (whatever the product gave, NaN from padding included)
+#pragma unroll
+        for (int kb = 0; kb < KBN; ++kb) {
+          const uint32_t rm = row_mask(lo[qb] - (k0 + kb * 32), hi[qb] - (k0 + kb * 32), h);
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[qb][kb][i] = keep_or_neg_inf(s[qb][kb][i], keep_bits(rm, i));
+        }
+      }
       float mx = -INFINITY;
-      if (interior) {
+      {
         float mk[KBN];   // one chain per key block, so that consecutive instructions are independent
 #pragma unroll
         for (int kb = 0; kb < KBN; ++kb) mk[kb] = -INFINITY;
@@ -364,14 +374,6 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
           for (int kb = 0; kb < KBN; ++kb) mk[kb] = fast_max3(mk[kb], s[qb][kb][i], s[qb][kb][i + 1]);
 #pragma unroll
         for (int kb = 0; kb < KBN; ++kb) mx = fast_max(mx, mk[kb]);
-      } else {
-#pragma unroll
-        for (int kb = 0; kb < KBN; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int key = k0 + kb * 32 + crow(i, h);
-            mx = (key >= lo[qb] && key < hi[qb]) ? fast_max(mx, s[qb][kb][i]) : mx;
-          }
       }
       mx = half_max(mx) * sl2e;
       const bool move = mx > m_run[qb] + kRescaleGap;
@@ -389,15 +391,6 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
       for (int kb = 0; kb < KBN; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[qb][kb][i] = fast_exp2(__builtin_fmaf(s[qb][kb][i], sl2e, -m_use));
-      if (!interior) {
-#pragma unroll
-        for (int kb = 0; kb < KBN; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int key = k0 + kb * 32 + crow(i, h);
-            s[qb][kb][i] = (key >= lo[qb] && key < hi[qb]) ? s[qb][kb][i] : 0.0f;
-          }
-      }
       float rs[2] = {0.0f, 0.0f};
 #pragma unroll
       for (int kb = 0; kb < KBN; ++kb) {
