@@ -12,13 +12,16 @@
  *     NULL = the default stream) and returns.
  *   - q/k/v/dO/o inputs are [B,H,T,D] with element strides given as int64[4]
  *     (batch, head, time, dim).  The dim stride must be 1; base pointers must be
- *     16-byte aligned and the other strides multiples of 16 bytes.  Outputs are
+ *     16-byte aligned and the other strides multiples of 16 bytes.  Rows of one
+ *     (batch, head) slice are addressed with 32-bit element offsets: the time stride must
+ *     be >= 0 and (T + 1024) * time_stride < 2^32, else SA_ERR_TOO_LARGE.  Outputs are
  *     written contiguous [B,H,T,D] (lse/delta: contiguous [B,H,T] float32).
  *   - dtype: 0 = float32, 1 = float16, 2 = bfloat16.  D in {16,32,64,128,256}.
  *   - lens: int32 per batch entry (may be NULL = every sequence has length T);
  *     lens_stride in elements; values are clamped to [0, T].
  *   - Outputs are fully written, including the zeros at positions t >= lens[b];
- *     the caller need not clear them first.
+ *     the caller need not clear them first.  Input positions t >= lens[b] are never
+ *     read, so they may hold anything.
  *   - Return value: 0 on success, > 0 a hipError_t from the launch, < 0 one of SA_ERR_*.
  *   - Re-entrant; no global mutable state apart from one-time kernel attribute set-up.
  */

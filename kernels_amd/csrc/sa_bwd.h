@@ -101,7 +101,7 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(const BwdParams p) {
   Frag qf[NF], gf[NF];
   float lse_q, delta_q;
   {
-    const int qr = qrow < T_ ? qrow : T_ - 1;
+    const int qr = qrow < L ? qrow : L - 1;
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh +
                   (int64_t)qr * p.q_st;
     const T* gp = reinterpret_cast<const T*>(p.d_o) + (int64_t)b * p.do_sb + (int64_t)hd * p.do_sh +
@@ -127,8 +127,8 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(const BwdParams p) {
     for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
 
   Stager<T, D, TK, NT> sk, sv;
-  sk.load(kbase, p.k_st, kt0 * TK, T_ - 1, tid);
-  sv.load(vbase, p.v_st, kt0 * TK, T_ - 1, tid);
+  sk.load(kbase, p.k_st, kt0 * TK, L - 1, tid);
+  sv.load(vbase, p.v_st, kt0 * TK, L - 1, tid);
   sk.store(smem, tid);
   sv.store(smem + TILE, tid);
   wait_all_loads();
@@ -140,8 +140,8 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(const BwdParams p) {
     const T* Vt = Kt + TILE;
     const bool more = t + 1 < kt1;
     if (more) {
-      sk.load(kbase, p.k_st, (t + 1) * TK, T_ - 1, tid);
-      sv.load(vbase, p.v_st, (t + 1) * TK, T_ - 1, tid);
+      sk.load(kbase, p.k_st, (t + 1) * TK, L - 1, tid);
+      sv.load(vbase, p.v_st, (t + 1) * TK, L - 1, tid);
     }
     const int k0 = t * TK;
     const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
 
   Frag kf[NF], vf[NF];
   {
-    const int kr = krow < T_ ? krow : T_ - 1;
+    const int kr = krow < L ? krow : L - 1;
     const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh +
                   (int64_t)kr * p.k_st;
     const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh +
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   auto load_rows = [&](int row0) {
     if (tid < TQ) {
       int r = row0 + tid;
-      r = r < T_ ? r : T_ - 1;
+      r = r < L ? r : L - 1;
       r_lse = lse_base[r];
       r_delta = delta_base[r];
     }
@@ -296,8 +296,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   };
   static_assert(TQ <= NW * 64, "one thread per staged row");
 
-  sq.load(qbase, p.q_st, qt0 * TQ, T_ - 1, tid);
-  sg.load(gbase, p.do_st, qt0 * TQ, T_ - 1, tid);
+  sq.load(qbase, p.q_st, qt0 * TQ, L - 1, tid);
+  sg.load(gbase, p.do_st, qt0 * TQ, L - 1, tid);
   load_rows(qt0 * TQ);
   store_stage(0);
   wait_all_loads();
@@ -311,8 +311,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
     const float* delta_t = lse_t + TQ;
     const bool more = t + 1 < qt1;
     if (more) {
-      sq.load(qbase, p.q_st, (t + 1) * TQ, T_ - 1, tid);
-      sg.load(gbase, p.do_st, (t + 1) * TQ, T_ - 1, tid);
+      sq.load(qbase, p.q_st, (t + 1) * TQ, L - 1, tid);
+      sg.load(gbase, p.do_st, (t + 1) * TQ, L - 1, tid);
       load_rows((t + 1) * TQ);
     }
     const int qs = t * TQ;
@@ -438,8 +438,8 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh;
   const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh;
   Loader ldk, ldv;
-  ldk.init(kbase, p.k_st, kt0 * TK, T_ - 1, wave, lane);
-  ldv.init(vbase, p.v_st, kt0 * TK, T_ - 1, wave, lane);
+  ldk.init(kbase, p.k_st, kt0 * TK, L - 1, wave, lane);
+  ldv.init(vbase, p.v_st, kt0 * TK, L - 1, wave, lane);
   auto issue_tile = [&](int t) {   // tiles are issued in ascending order
     T* st = smem + ((t - kt0) % NST) * STAGE;
     ldk.issue(st, wave);
@@ -454,7 +454,7 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
   Frag qf[NF], gf[NF];
   float lse_q, delta_q;
   {
-    const int qr = qrow < T_ ? qrow : T_ - 1;
+    const int qr = qrow < L ? qrow : L - 1;
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh +
                   (int64_t)qr * p.q_st;
     const T* gp = reinterpret_cast<const T*>(p.d_o) + (int64_t)b * p.do_sb + (int64_t)hd * p.do_sh +
@@ -593,14 +593,14 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
   const float* delta_base = p.delta + (int64_t)bh * T_;
   auto stage_ptr = [&](int t) { return smem_raw + ((t - qt0) % NST) * STAGE_BYTES; };
   Loader ldq, ldg;
-  ldq.init(qbase, p.q_st, qt0 * TQ, T_ - 1, wave, lane);
-  ldg.init(gbase, p.do_st, qt0 * TQ, T_ - 1, wave, lane);
+  ldq.init(qbase, p.q_st, qt0 * TQ, L - 1, wave, lane);
+  ldg.init(gbase, p.do_st, qt0 * TQ, L - 1, wave, lane);
   auto issue_tile = [&](int t) {   // tiles are issued in ascending order
     T* st = reinterpret_cast<T*>(stage_ptr(t));
     // lanes [0, RPW) fetch lse, lanes [RPW, 2*RPW) fetch delta of this wave's RPW rows
     if (lane < 2 * RPW) {
       int r = t * TQ + wave * RPW + (lane % RPW);
-      r = r < T_ ? r : T_ - 1;
+      r = r < L ? r : L - 1;
       const float* src = (lane < RPW ? lse_base : delta_base) + r;
       float* dst = reinterpret_cast<float*>(stage_ptr(t) + 2 * TILE * sizeof(T)) + wave * 2 * RPW;
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
@@ -617,7 +617,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
 
   Frag kf[NF], vf[NF];
   {
-    const int kr = krow < T_ ? krow : T_ - 1;
+    const int kr = krow < L ? krow : L - 1;
     const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh +
                   (int64_t)kr * p.k_st;
     const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh +

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
   // ---- Q fragments stay in registers for the whole key loop -------------------------
   Frag qf[NF];
   {
-    const int qr = qrow < T_ ? qrow : T_ - 1;
+    const int qr = qrow < L ? qrow : L - 1;
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh +
                   (int64_t)qr * p.q_st;
 #pragma unroll
@@ -94,8 +94,8 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
   float m_run = -INFINITY, l_run = 0.0f;
 
   Stager<T, D, TK, NT> sk, sv;
-  sk.load(kbase, p.k_st, kt0 * TK, T_ - 1, tid);
-  sv.load(vbase, p.v_st, kt0 * TK, T_ - 1, tid);
+  sk.load(kbase, p.k_st, kt0 * TK, L - 1, tid);
+  sv.load(vbase, p.v_st, kt0 * TK, L - 1, tid);
   sk.store(smem, tid);
   sv.store(smem + TILE, tid);
   wait_all_loads();
@@ -107,8 +107,8 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
     const T* Vt = Kt + TILE;
     const bool more = t + 1 < kt1;
     if (more) {
-      sk.load(kbase, p.k_st, (t + 1) * TK, T_ - 1, tid);
-      sv.load(vbase, p.v_st, (t + 1) * TK, T_ - 1, tid);
+      sk.load(kbase, p.k_st, (t + 1) * TK, L - 1, tid);
+      sv.load(vbase, p.v_st, (t + 1) * TK, L - 1, tid);
     }
     const int k0 = t * TK;
 
@@ -287,8 +287,8 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh;
   const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.v_sb + (int64_t)hd * p.v_sh;
   Loader ldk, ldv;
-  ldk.init(kbase, p.k_st, kt0 * TK, T_ - 1, wave, lane);
-  ldv.init(vbase, p.v_st, kt0 * TK, T_ - 1, wave, lane);
+  ldk.init(kbase, p.k_st, kt0 * TK, L - 1, wave, lane);
+  ldv.init(vbase, p.v_st, kt0 * TK, L - 1, wave, lane);
   auto issue_tile = [&](int t) {   // tiles are issued in ascending order
     T* st = smem + ((t - kt0) % NST) * STAGE;
     ldk.issue(st, wave);
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   Frag qf[QB][NF];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    const int qr = qrow[qb] < T_ ? qrow[qb] : T_ - 1;
+    const int qr = qrow[qb] < L ? qrow[qb] : L - 1;
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh +
                   (int64_t)qr * p.q_st;
 #pragma unroll

@@ -175,6 +175,29 @@ def test_softmax_scale(scale, dtype):
     check_against_dense(q, k, v, d_o, lens, C, R, dtype, sm_scale=scale)
 
 
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 32), (torch.float16, 64), (torch.bfloat16, 128), (torch.bfloat16, 256)])
+@pytest.mark.parametrize("T,C,R", [(150, 16, 2), (300, 64, 1), (520, 256, 0)])
+def test_padding_is_never_read(T, C, R, dtype, D):
+    """Positions t >= lens[b] of q, k, v and dO may hold anything (the reference masks its loads,
+    kernel.py:246-274): NaN there must give bit-identical results to zeros there."""
+    B, H = 3, 2
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=27, dtype=dtype)
+    lens = torch.tensor([T - 1, max(T // 2 - 3, 1), 37], dtype=torch.int32)
+    clean, dirty = [], []
+    for t in (q, k, v, d_o):
+        z, n = t.clone(), t.clone()
+        for b in range(B):
+            z[b, :, int(lens[b]):] = 0
+            n[b, :, int(lens[b]):] = float("nan")
+        clean.append(z)
+        dirty.append(n)
+    want = run_kernel(*clean, lens, C, R)
+    got = run_kernel(*dirty, lens, C, R)
+    for name, a, b in zip(("O", "LSE", "dQ", "dK", "dV"), got, want):
+        assert torch.isfinite(a).all(), f"{name}: padding leaked into the result"
+        assert torch.equal(a, b), f"{name}: result depends on the padded positions"
+
+
 def test_empty_inputs_and_zero_lengths():
     from streaming_attention import streaming_attention
 
