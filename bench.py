@@ -53,7 +53,7 @@ def unmasked_pairs(T, C, R, lens_list):
     return total
 
 
-def make_inputs(name, device):
+def make_inputs(name, device, zeros=False):
     import torch
 
     B, H, T, D, dtype_name, C, R, lens_mode, qkv_scale = WORKLOADS[name]
@@ -78,6 +78,8 @@ def make_inputs(name, device):
     q, k, v = [(torch.randn(B, H, T, D, generator=dg, device=device, dtype=torch.float32) * scale).to(dtype)
                for _ in range(3)]
     d_o = torch.randn(B, H, T, D, generator=dg, device=device, dtype=torch.float32).to(dtype)
+    if zeros:   # same launches on operands that never toggle a multiplier input
+        q, k, v, d_o = (torch.zeros_like(t) for t in (q, k, v, d_o))
     return dict(q=q, k=k, v=v, d_o=d_o, lens=lens.to(device) if lens is not None else None,
                 lens_list=lens_list, B=B, H=H, T=T, D=D, C=C, R=R, dtype=dtype_name)
 
@@ -166,6 +168,55 @@ HBM_BYTES_PER_LAUNCH = {
 }
 
 
+def reference_sweep(device, iters=20):
+    """The reference's own benchmark grid (benchmark/benchmark_streaming_attention.py:113-292):
+    fp16, B=128, H=12, D=64, (context, back) in {(10, 9), (32, 2)}, six lengths from 257 to 3000,
+    lens = None; forward under inference mode and forward+backward, HIP-event means, and the
+    reference's flop count 4*T*W*H*D*B with W = context*(1+back) (x3.5 for forward+backward), which
+    counts the full band, not the unmasked pairs."""
+    import torch
+    from streaming_attention import streaming_attention
+
+    B, H, D = 128, 12, 64
+    rows = []
+    for C, R in ((10, 9), (32, 2)):
+        for T in [int(round(257 + i * (3000 - 257) / 5)) for i in range(6)]:
+            g = torch.Generator(device=device).manual_seed(20)
+            q, k, v = [torch.randn(B, H, T, D, generator=g, device=device, dtype=torch.float16) for _ in range(3)]
+            d_o = torch.randn(B, H, T, D, generator=g, device=device, dtype=torch.float16)
+
+            def timed(fn):
+                for _ in range(3):
+                    fn()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(iters):
+                    fn()
+                e1.record()
+                e1.synchronize()
+                return e0.elapsed_time(e1) / iters
+
+            def fwd():
+                with torch.inference_mode():
+                    streaming_attention(q, k, v, None, C, R)
+
+            qg, kg, vg = (t.clone().requires_grad_() for t in (q, k, v))
+
+            def fwd_bwd():
+                qg.grad = kg.grad = vg.grad = None
+                streaming_attention(qg, kg, vg, None, C, R).backward(d_o)
+
+            t_f, t_fb = timed(fwd), timed(fwd_bwd)
+            band = 4.0 * T * C * (1 + R) * H * D * B
+            rows.append({"context_size": C, "back_contexts": R, "T": T, "fwd_ms": t_f, "fwd_bwd_ms": t_fb,
+                         "fwd_band_tflops": band / (t_f * 1e-3) / 1e12,
+                         "fwd_bwd_band_tflops": 3.5 * band / (t_fb * 1e-3) / 1e12,
+                         "unmasked_pairs_per_head": unmasked_pairs(T, C, R, [T] * B)})
+            del q, k, v, d_o, qg, kg, vg
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -176,6 +227,11 @@ def main():
     ap.add_argument("--kernel-iters", type=int, default=10)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy (known traffic) for scaling HBM counters")
+    ap.add_argument("--zero-inputs", action="store_true",
+                    help="all-zero q, k, v, dO: the same kernels and launch shapes without data-dependent "
+                         "switching power (a diagnostic; the result line is marked and is not the metric)")
+    ap.add_argument("--reference-sweep", action="store_true",
+                    help="time the grid of the reference's own benchmark script instead of a workload")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -193,7 +249,11 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "3 copies of 1 GiB (2^28 fp32): 1048576 KiB read and written each"}))
         return
-    w = make_inputs(args.workload, dev)
+    if args.reference_sweep:
+        print(json.dumps({"sweep": "reference benchmark grid, fp16 B=128 H=12 D=64", "n_gpus": 1,
+                          "rows": reference_sweep(dev)}))
+        return
+    w = make_inputs(args.workload, dev, zeros=args.zero_inputs)
     B, H, T, D, C, R = w["B"], w["H"], w["T"], w["D"], w["C"], w["R"]
     P = unmasked_pairs(T, C, R, w["lens_list"])
     flops_step = 14.0 * D * H * P
@@ -226,7 +286,7 @@ def main():
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"bfloat16": "bf16", "float16": "f16", "float32": "f32"}[w["dtype"]],
-        "data": "synthetic",
+        "data": "synthetic, all zeros (diagnostic run)" if args.zero_inputs else "synthetic",
         "config": {"workload": args.workload, "B": B, "H": H, "T": T, "D": D, "context_size": C,
                    "back_contexts": R, "lens": w["lens_list"], "unmasked_pairs_per_head": P,
                    "flops_per_step": flops_step},
