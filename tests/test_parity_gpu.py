@@ -198,6 +198,63 @@ def test_padding_is_never_read(T, C, R, dtype, D):
         assert torch.equal(a, b), f"{name}: result depends on the padded positions"
 
 
+def _random_case(seed):
+    rng = np.random.default_rng(1000 + seed)
+    D = int(rng.choice([16, 32, 64, 64, 128, 128, 256]))
+    dtype = [torch.float32, torch.float16, torch.bfloat16][int(rng.integers(0, 3))]
+    B, H = int(rng.integers(1, 5)), int(rng.integers(1, 4))
+    T = int(rng.choice([1, 2, 31, 32, 33, 63, 64, 65, 127, 129, 255, 257, 300, 511, 640]))
+    C = int(rng.choice([1, 2, 7, 16, 31, 32, 33, 64, 100, 128, 256, 10**6]))
+    R = int(rng.choice([0, 0, 1, 2, 3, 8, 17, 10**6]))
+    lens = None
+    if rng.random() < 0.75:
+        lens = torch.tensor(rng.integers(0, T + 3, B), dtype=torch.int32)
+    scale = None if rng.random() < 0.5 else float(rng.choice([-1.0, 1.0]) * rng.uniform(0.02, 0.2))
+    bthd = bool(rng.random() < 0.4)
+    return B, H, T, D, C, R, lens, dtype, scale, bthd
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_problems(seed):
+    """Seeded random draws over every axis at once: head dim, dtype, batch, heads, lengths around the
+    tile sizes, chunk sizes that do and do not divide the tiles, unbounded windows, lens of 0 and
+    beyond T, explicit and negative scales, [B,T,H,D]-stored inputs."""
+    from streaming_attention import streaming_attention
+
+    B, H, T, D, C, R, lens, dtype, scale, bthd = _random_case(seed)
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=500 + seed, dtype=dtype)
+    if dtype != torch.float32 and scale is not None:
+        scale = scale * 0.5   # keeps gradient magnitudes inside the absolute part of the 16-bit bar
+    dev = torch.device("cuda:0")
+
+    def place(t):
+        t = t.to(dev)
+        return (t.transpose(1, 2).contiguous().transpose(1, 2) if bthd else t).requires_grad_()
+
+    qd, kd, vd = place(q), place(k), place(v)
+    kw = {} if scale is None else {"sm_scale": scale}
+    out, lse = streaming_attention(qd, kd, vd, lens.to(dev) if lens is not None else None, C, R,
+                                   return_lse=True, **kw)
+    out.backward(d_o.to(dev))
+    ref = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=scale, d_out=d_o)
+    assert_close("O", out, ref["O"], dtype)
+    assert_close("LSE", lse, ref["LSE"], dtype)
+    assert_close("dQ", qd.grad, ref["dQ"], dtype)
+    assert_close("dK", kd.grad, ref["dK"], dtype)
+    assert_close("dV", vd.grad, ref["dV"], dtype)
+
+
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 256)])
+def test_results_are_deterministic(dtype, D):
+    """No atomics and a fixed reduction order: two runs on the same inputs agree bit for bit."""
+    q, k, v, d_o = make_inputs(2, 3, 333, D, seed=28, dtype=dtype)
+    lens = torch.tensor([333, 170], dtype=torch.int32)
+    first = run_kernel(q, k, v, d_o, lens, 48, 2)
+    second = run_kernel(q, k, v, d_o, lens, 48, 2)
+    for name, a, b in zip(("O", "LSE", "dQ", "dK", "dV"), first, second):
+        assert torch.equal(a, b), name
+
+
 def test_empty_inputs_and_zero_lengths():
     from streaming_attention import streaming_attention
 
