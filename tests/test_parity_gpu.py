@@ -312,7 +312,7 @@ def test_c_abi_direct_calls():
                           s4(q), s4(k), s4(v), B, H, T, D, C, R, sc, 2, st) == -4
 
 
-# ---- BASELINE.json configurations at their real shapes -------------------------------
+# ---- the benchmark configurations at their real shapes --------------------------------
 
 def _lens_for(mode, B, T, g):
     if mode == "full":
