@@ -139,6 +139,28 @@ def test_noncontiguous_inputs(dtype):
         assert_close("dV", vd.grad, ref["dV"], dtype)
 
 
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float32, 32)])
+def test_packed_qkv_projection_is_read_in_place(dtype, D):
+    """q, k, v as views of one [B, T, 3, H, D] projection output: no copies on the way in, and the
+    gradient arrives in the packed tensor."""
+    from streaming_attention import streaming_attention
+    from streaming_attention.ops import _kernel_layout
+
+    dev = torch.device("cuda:0")
+    B, H, T, C, R = 2, 3, 200, 64, 1
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=29, dtype=dtype)
+    lens = torch.tensor([200, 77], dtype=torch.int32)
+    qkv = torch.stack([t.transpose(1, 2) for t in (q, k, v)], dim=2).to(dev).requires_grad_()   # [B,T,3,H,D]
+    views = [qkv[:, :, i].transpose(1, 2) for i in range(3)]                                    # [B,H,T,D]
+    assert all(_kernel_layout(x) is x and not x.is_contiguous() for x in views)
+    out = streaming_attention(*views, lens.to(dev), C, R)
+    out.backward(d_o.to(dev))
+    ref = sa_oracle.dense_f64(q, k, v, lens, C, R, d_out=d_o)
+    assert_close("O", out, ref["O"], dtype)
+    for i, name in enumerate(("dQ", "dK", "dV")):
+        assert_close(name, qkv.grad[:, :, i].transpose(1, 2), ref[name], dtype)
+
+
 def test_backward_op_accepts_foreign_gradient_and_missing_lse():
     """The backward dispatcher op on its own: fp32 strided dO with fp16 q/k/v
     (tests/test_streaming_attention.py:224-248) and an empty lse (forward without return_lse)."""
