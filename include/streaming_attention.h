@@ -13,8 +13,8 @@
  *   - q/k/v/dO/o inputs are [B,H,T,D] with element strides given as int64[4]
  *     (batch, head, time, dim).  The dim stride must be 1; base pointers must be
  *     16-byte aligned and the other strides multiples of 16 bytes.  Rows of one
- *     (batch, head) slice are addressed with 32-bit element offsets: the time stride must
- *     be >= 0 and (T + 1024) * time_stride < 2^32, else SA_ERR_TOO_LARGE.  Outputs are
+ *     (batch, head) slice are addressed with 32-bit byte offsets: the time stride must
+ *     be >= 0 and (T + 1024) * time_stride * element_size < 2^32, else SA_ERR_TOO_LARGE.  Outputs are
  *     written contiguous [B,H,T,D] (lse/delta: contiguous [B,H,T] float32).
  *   - dtype: 0 = float32, 1 = float16, 2 = bfloat16.  D in {16,32,64,128,256}.
  *   - lens: int32 per batch entry (may be NULL = every sequence has length T);

@@ -12,7 +12,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // strides are element counts; dim stride 1, the others whole 16-byte vectors
-// and the kernels address rows of one (batch, head) slice with 32-bit element offsets
+// and the kernels address rows of one (batch, head) slice with 32-bit byte offsets
 int check_layout(const void* p, const int64_t* s, int dtype, int T) {
   if (!p || !s) return SA_ERR_ARG;
   const int64_t vec = dtype == SA_DTYPE_F32 ? 4 : 8;
@@ -21,7 +21,7 @@ int check_layout(const void* p, const int64_t* s, int dtype, int T) {
   for (int i = 0; i < 3; ++i)
     if (s[i] % vec != 0) return SA_ERR_LAYOUT;
   if (s[2] < 0) return SA_ERR_LAYOUT;
-  if (((int64_t)T + 1024) * s[2] >= (int64_t(1) << 32)) return SA_ERR_TOO_LARGE;
+  if (((int64_t)T + 1024) * s[2] * (dtype == SA_DTYPE_F32 ? 4 : 2) >= (int64_t(1) << 32)) return SA_ERR_TOO_LARGE;
   return SA_OK;
 }
 

@@ -410,17 +410,14 @@ SA_DEV void mma_tr_n(f32x16 (&acc)[NQ][NM], const T* X, int rb, const typename E
 }
 
 // Asynchronous copy of [ROWS][D] row-major global tiles into swizzled LDS tiles with
-// global_load_lds_dwordx4: the data never passes through registers.  One instruction moves
+// buffer_load_dwordx4 ... lds: the data never passes through registers.  One instruction moves
 // 1 KiB (64 lanes x 16 bytes) to consecutive LDS addresses, i.e. 1024/(2*D) whole rows; lane l
 // therefore fetches, for physical chunk l % CPR of its row, the logical chunk that the swizzle
 // maps there.  The NW waves of a workgroup interleave instruction by instruction.  Completion
 // is tracked by vmcnt; visibility to the other waves needs a barrier after the wait.
 //
-// Tiles are issued in ascending order.  The object keeps, per lane, the 32-bit element offset
-// of its row in the next tile, so that issuing costs an add, a clamp and an add per
-// instruction and no multiplication; rows past the end of the sequence are clamped to the
-// last row (their contents are masked by the caller).  Offsets are 32-bit: the host checks
-// that T * row_stride fits.
+// Tiles are issued in ascending order.  Offsets are 32-bit byte offsets inside one (batch, head)
+// slice: the host checks that T * row_stride * sizeof(T) fits.
 template <typename T, int D, int ROWS, int NW> struct AsyncTile {
   using G_ = TileGeom<T, D>;
   static_assert(G_::SWZ, "asynchronous tiles use the swizzled layout");
@@ -431,38 +428,39 @@ template <typename T, int D, int ROWS, int NW> struct AsyncTile {
   static_assert((RPI * NW) % 16 == 0, "the swizzle of a lane must not depend on the instruction");
   static constexpr int PER_WAVE = NI / NW;                  // instructions per wave per tile
 
-  const T* base;      // wave-uniform: first element of this (batch, head)
-  uint32_t rowoff;    // element offset of this lane's row (instruction 0) in the next tile
-  uint32_t coloff;    // swizzled column offset of this lane, in elements
-  uint32_t last;      // element offset of the last valid row
-  uint32_t istep;     // offset between rows of consecutive instructions of one wave
-  uint32_t tstep;     // offset between consecutive tiles
+  // Buffer addressing: a resource descriptor for the (batch, head) slice whose extent ends with
+  // the last valid row, one per-lane byte offset that never changes, and a scalar byte offset
+  // that carries the tile and the instruction.  No vector arithmetic per load, and rows past
+  // the last valid one come back as zeros from the hardware's range check.
+  __amdgpu_buffer_rsrc_t rsrc;
+  uint32_t voff;      // byte offset of this lane's 16 bytes inside instruction 0 of tile 0
+  uint32_t soff;      // wave-uniform byte offset of the next tile
+  uint32_t istep;     // bytes between rows of consecutive instructions of one wave
+  uint32_t tstep;     // bytes between consecutive tiles
 
   SA_DEV void init(const T* gbase, int64_t row_stride, int first_row, int last_row, int wave, int lane) {
+    constexpr uint32_t ES = (uint32_t)sizeof(T);
     const int lrow = lane / G_::CPR, pch = lane % G_::CPR;
     const uint32_t rs = (uint32_t)row_stride;
-    base = gbase;
-    rowoff = (uint32_t)(first_row + wave * RPI + lrow) * rs;
-    coloff = (uint32_t)((pch ^ G_::swz(wave * RPI + lrow)) * Elem<T>::VEC);
-    last = (uint32_t)last_row * rs;
-    istep = (uint32_t)(NW * RPI) * rs;
-    tstep = (uint32_t)ROWS * rs;
+    const uint32_t bytes = ((uint32_t)last_row * rs + (uint32_t)D) * ES;
+    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gbase), 0, (int)bytes, 0x00020000);
+    voff = ((uint32_t)(wave * RPI + lrow) * rs + (uint32_t)((pch ^ G_::swz(wave * RPI + lrow)) * Elem<T>::VEC)) * ES;
+    soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)first_row * rs * ES));
+    istep = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(NW * RPI) * rs * ES));
+    tstep = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)ROWS * rs * ES));
   }
   // instructions [I0, I1) of this wave's share of the next tile
   template <int I0, int I1> SA_DEV void issue_part(T* tile, int wave) const {
     static_assert(0 <= I0 && I0 <= I1 && I1 <= PER_WAVE, "instruction range");
 #pragma unroll
     for (int i = I0; i < I1; ++i) {
-      uint32_t ro = rowoff + (uint32_t)i * istep;
-      ro = ro < last ? ro : last;
-      const T* src = base + (ro + coloff);
       T* dst = tile + (i * NW + wave) * RPI * D;           // wave-uniform
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (SA_LDS void*)dst, 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (SA_LDS void*)dst, 16, (int)voff,
+                                               (int)(soff + (uint32_t)i * istep), 0, 0);
     }
   }
   SA_DEV void issue(T* tile, int wave) const { issue_part<0, PER_WAVE>(tile, wave); }
-  SA_DEV void advance() { rowoff += tstep; }
+  SA_DEV void advance() { soff += tstep; }
 };
 
 // s_waitcnt vmcnt(N), other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and 15:14).

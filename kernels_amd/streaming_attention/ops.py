@@ -30,14 +30,14 @@ def _kernel_layout(t: torch.Tensor) -> torch.Tensor:
     """Return ``t`` itself when the kernels can read it in place (unit stride along the head
     dimension, every other stride and the base address a multiple of 16 bytes), otherwise a
     contiguous copy.  The kernels address the rows of one (batch, head) slice with 32-bit
-    offsets (a contiguous tensor is within that range up to tens of millions of positions)."""
+    byte offsets (a contiguous tensor is within that range up to tens of millions of positions)."""
     es = t.element_size()
     vec = _VEC_BYTES // es
     ok = (
         t.stride(-1) == 1
         and all(s % vec == 0 for s in t.stride()[:-1])
         and t.data_ptr() % _VEC_BYTES == 0
-        and (t.shape[-2] + 1024) * t.stride(-2) < 2**32
+        and (t.shape[-2] + 1024) * t.stride(-2) * es < 2**32
     )
     return t if ok else t.contiguous()
 
