@@ -107,6 +107,10 @@ int sa_backward(const void* q, const void* k, const void* v,
  *          2: forward key tile (16-bit types)   3: forward key tile (fp32)
  *          4: dQ key tile          5: dK/dV query tile
  *          6: queries (or keys) owned by one workgroup
+ *      (1-6 describe the kernels used for float32 and for D in {16, 32, 256})
+ *          7, 8: waves per workgroup of the wide / narrow forward and dQ kernels used for the
+ *                16-bit types at D in {64, 128} (each wave owns 32 queries)
+ *          9: smallest context_size for which the wide kernels are chosen
  *   anything else: -1 */
 int sa_query(int what);
 

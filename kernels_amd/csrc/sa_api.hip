@@ -171,6 +171,9 @@ int sa_query(int what) {
     case 4: return Cfg<__bf16>::DQ_TK;
     case 5: return Cfg<__bf16>::DKDV_TQ;
     case 6: return Cfg<__bf16>::NW * 32;
+    case 7: return Cfg<__bf16>::WIDE_NW;
+    case 8: return Cfg<__bf16>::NARROW_NW;
+    case 9: return Cfg<__bf16>::WIDE_CHUNK;
   }
   return -1;
 }

@@ -44,7 +44,8 @@ template <typename T> struct Cfg {
   // workgroup's queries lie in one chunk; with smaller chunks the union of the waves'
   // windows grows and 4 waves (128 queries) waste less of every tile.
   static constexpr int WIDE_NW = 8, NARROW_NW = 4;
-  static constexpr bool wide(int chunk) { return chunk >= 256; }
+  static constexpr int WIDE_CHUNK = 256;
+  static constexpr bool wide(int chunk) { return chunk >= WIDE_CHUNK; }
   static constexpr int DQ2_TK = SA_DQ2_TK, DQ2_NST = SA_DQ2_NST;
   static constexpr int DKDV2_NW = SA_DKDV2_NW, DKDV2_TQ = SA_DKDV2_TQ, DKDV2_NST = SA_DKDV2_NST;
   static constexpr int FWD2_QB = SA_FWD2_QB;

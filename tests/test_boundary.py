@@ -42,6 +42,7 @@ def test_query_and_error_strings(lib):
     assert lib.sa_query(0) >= 1
     assert lib.sa_query(1) in (4, 8)
     assert lib.sa_query(2) % 32 == 0 and lib.sa_query(3) % 32 == 0
+    assert (lib.sa_query(7), lib.sa_query(8)) == (8, 4) and lib.sa_query(9) == 256
     assert lib.sa_query(99) == -1
     assert b"success" in lib.sa_error_string(0)
     for code in (-1, -2, -3, -4, -5):
