@@ -402,6 +402,18 @@ def test_baseline_configs_full_size(name, B, H, T, D, dtype, C, R, lens_mode, qk
     out2.backward(d_o)
     assert torch.equal(out, out2) and torch.equal(q.grad, q2.grad) and torch.equal(k.grad, k2.grad)
     assert torch.equal(v.grad, v2.grad)
+    # the backward pass is linear in dO: doubling dO (exact in binary floating point) doubles every
+    # gradient bit for bit, and a zero dO gives exactly zero
+    q5, k5, v5 = (t.detach().clone().requires_grad_() for t in (q, k, v))
+    streaming_attention(q5, k5, v5, ld, C, R).backward(d_o * 2)
+    for got, base in ((q5.grad, q.grad), (k5.grad, k.grad), (v5.grad, v.grad)):
+        if dtype == torch.float16:   # fp16 intermediates reach the subnormal range, where rounding does not scale
+            assert torch.allclose(got.float(), base.float() * 2, atol=2e-3, rtol=1e-2)
+        else:
+            assert torch.equal(got, base * 2)
+    q6, k6, v6 = (t.detach().clone().requires_grad_() for t in (q, k, v))
+    streaming_attention(q6, k6, v6, ld, C, R).backward(torch.zeros_like(d_o))
+    assert not bool(q6.grad.any()) and not bool(k6.grad.any()) and not bool(v6.grad.any())
     if B > 1:
         # batch entries are independent: reversing the batch reverses the outputs bit for bit
         perm = torch.arange(B - 1, -1, -1, device=dev)
