@@ -514,14 +514,17 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
     }
   }
 
-  if (qrow < T_) {
-    if (qrow >= L) {
+  if (qrow >= L) {
 #pragma unroll
-      for (int m = 0; m < DB; ++m)
+    for (int m = 0; m < DB; ++m)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
-    }
-    store_acc_T<T, D, DB>(dq_base + (int64_t)qrow * D, acc, -p.scale, h);
+      for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
+  }
+  __syncthreads();   // the row patches lie over the tile stages
+  {
+    T* patch = smem + wave * RowPatch<T, D>::ELEMS;
+    const int row0 = q0 + wave * 32;
+    store_rows_coalesced<T, D, DB>(patch, dq_base + (int64_t)row0 * D, T_ - row0, acc, -p.scale, lane);
   }
 }
 
@@ -694,15 +697,19 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
     }
   }
 
-  if (krow < T_) {
-    if (krow >= L) {
+  if (krow >= L) {
 #pragma unroll
-      for (int m = 0; m < DB; ++m)
+    for (int m = 0; m < DB; ++m)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
-    }
-    store_acc_T<T, D, DB>(dk_base + (int64_t)krow * D, dk, -p.scale, h);
-    store_acc_T<T, D, DB>(dv_base + (int64_t)krow * D, dv, 1.0f, h);
+      for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
+  }
+  // the row patches lie over the tile stages: wait until no wave reads the last tile any more
+  __syncthreads();
+  {
+    T* patch = reinterpret_cast<T*>(smem_raw) + wave * RowPatch<T, D>::ELEMS;
+    const int row0 = k0 + wave * 32;
+    store_rows_coalesced<T, D, DB>(patch, dk_base + (int64_t)row0 * D, T_ - row0, dk, -p.scale, lane);
+    store_rows_coalesced<T, D, DB>(patch, dv_base + (int64_t)row0 * D, T_ - row0, dv, 1.0f, lane);
   }
 }
 

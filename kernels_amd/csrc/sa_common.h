@@ -562,6 +562,38 @@ SA_DEV void store_acc_T(T* row_ptr, const f32x16 (&acc)[DB], float mul, int h) {
     }
 }
 
+// The same store through a wave-private LDS patch, so that global memory sees whole rows: the
+// accumulators hold X^T (a lane owns one row, four consecutive d per register group), which
+// stored directly puts 8 bytes per lane on 32 different rows per instruction.  Here the lane
+// writes its row into the patch, and the wave reads it back four rows at a time, 16 lanes x 16
+// bytes per row, for 1 KiB stores of contiguous rows.  16-bit types only.
+template <typename T, int D> struct RowPatch {
+  static constexpr int PITCH = D + 8;              // elements: rows stay 16-byte aligned, 4 banks apart
+  static constexpr int ELEMS = 32 * PITCH;         // per wave
+  static constexpr int CPR = D / 8;                // 16-byte chunks per row
+  static constexpr int RPI = 64 / CPR;             // rows per store instruction
+};
+template <typename T, int D, int DB>
+SA_DEV void store_rows_coalesced(T* patch, T* out_rows, int rows_valid, const f32x16 (&acc)[DB], float mul,
+                                 int lane) {
+  using P = RowPatch<T, D>;
+  static_assert(Elem<T>::HALF && DB * 32 == D, "16-bit types, one accumulator block per 32 columns");
+  const int c = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int m = 0; m < DB; ++m)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      store4<T>(patch + c * P::PITCH + m * 32 + 8 * g + 4 * h, acc[m][4 * g] * mul, acc[m][4 * g + 1] * mul,
+                acc[m][4 * g + 2] * mul, acc[m][4 * g + 3] * mul);
+  const int rr = lane / P::CPR, ch = lane % P::CPR;
+#pragma unroll
+  for (int j = 0; j < 32 / P::RPI; ++j) {
+    const int row = j * P::RPI + rr;
+    const u32x4 v16 = *reinterpret_cast<const u32x4*>(patch + row * P::PITCH + ch * 8);
+    if (row < rows_valid) *reinterpret_cast<u32x4*>(out_rows + (int64_t)row * D + ch * 8) = v16;
+  }
+}
+
 struct FwdParams {
   const void *q, *k, *v;
   void* o;          // contiguous [B,H,T,D]

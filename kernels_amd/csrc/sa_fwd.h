@@ -412,22 +412,23 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   }
 
   // ---- epilogue --------------------------------------------------------------------
+  __syncthreads();   // the row patches lie over the tile stages
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const float l_tot = half_sum(l_run[qb]);
     const bool valid = qrow[qb] < L;
-    if (qrow[qb] < T_) {
-      const float inv = valid ? 1.0f / l_tot : 0.0f;
-      if (!valid) {
+    const float inv = valid ? 1.0f / l_tot : 0.0f;
+    if (!valid) {
 #pragma unroll
-        for (int m = 0; m < DB; ++m)
+      for (int m = 0; m < DB; ++m)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) oacc[qb][m][i] = 0.0f;
-      }
-      store_acc_T<T, D, DB>(o_base + (int64_t)qrow[qb] * D, oacc[qb], inv, h);
-      if (lse_base && h == 0)
-        lse_base[qrow[qb]] = valid ? m_run[qb] + __builtin_amdgcn_logf(l_tot) : 0.0f;
+        for (int i = 0; i < 16; ++i) oacc[qb][m][i] = 0.0f;
     }
+    T* patch = smem + wave * RowPatch<T, D>::ELEMS;
+    const int row0 = q0 + wave * WQ + qb * 32;
+    store_rows_coalesced<T, D, DB>(patch, o_base + (int64_t)row0 * D, T_ - row0, oacc[qb], inv, lane);
+    if (lse_base && h == 0 && qrow[qb] < T_)
+      lse_base[qrow[qb]] = valid ? m_run[qb] + __builtin_amdgcn_logf(l_tot) : 0.0f;
   }
 }
 

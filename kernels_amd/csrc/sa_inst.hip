@@ -57,7 +57,10 @@ static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 template <int D, int NW> static int fwd2_launch(FwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   constexpr int TQ = NW * C::FWD2_QB * 32;
-  constexpr size_t lds = (size_t)C::FWD2_NST * 2 * C::FWD_TK * D * sizeof(ElemT);
+  // tile stages; the epilogue's row patches (one per wave) reuse the same memory
+  constexpr size_t stages = (size_t)C::FWD2_NST * 2 * C::FWD_TK * D * sizeof(ElemT);
+  constexpr size_t patches = (size_t)NW * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
+  constexpr size_t lds = stages > patches ? stages : patches;
   auto kern = fwd2_kernel<ElemT, D, C::FWD2_QB, NW, C::FWD_TK, C::FWD2_NST>;
   static std::once_flag once;
   if (int rc = prepare(kern, lds, once)) return rc;
@@ -106,7 +109,9 @@ template <> int launch_delta<ElemT, SA_DGROUP>(const DeltaParams& p, int D, hipS
 template <int D, int NW> static int dq2_launch(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   constexpr int TQ = NW * 32;
-  constexpr size_t lds = (size_t)C::DQ2_NST * 2 * C::DQ2_TK * D * sizeof(ElemT);
+  constexpr size_t stages = (size_t)C::DQ2_NST * 2 * C::DQ2_TK * D * sizeof(ElemT);
+  constexpr size_t patches = (size_t)NW * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
+  constexpr size_t lds = stages > patches ? stages : patches;
   auto kern = dq2_kernel<ElemT, D, NW, C::DQ2_TK, C::DQ2_NST>;
   static std::once_flag once;
   if (int rc = prepare(kern, lds, once)) return rc;
@@ -143,8 +148,10 @@ template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
     constexpr int TKB = C::DKDV2_NW * 32;
-    constexpr size_t lds =
+    constexpr size_t stages =
         (size_t)C::DKDV2_NST * (2 * C::DKDV2_TQ * D * sizeof(ElemT) + 2 * C::DKDV2_TQ * sizeof(float));
+    constexpr size_t patches = (size_t)C::DKDV2_NW * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
+    constexpr size_t lds = stages > patches ? stages : patches;
     auto kern = dkdv2_kernel<ElemT, D, C::DKDV2_NW, C::DKDV2_TQ, C::DKDV2_NST>;
     static std::once_flag once;
     if (int rc = prepare(kern, lds, once)) return rc;
