@@ -183,7 +183,7 @@ def cpu_baseline(w, name, budget_s=12.0):
 # what the same counters read for the 1 GiB copy of --calibrate-copy: x2.000 and x1.000).  Counter runs
 # cannot be made from inside a timed run, so the figures of the committed profile summary are quoted here.
 HBM_BYTES_PER_LAUNCH = {
-    "headline_bf16_T16384_D128": {"fwd": 1.686e9, "delta": 5.411e8, "dq": 2.063e9, "dkdv": 1.718e9},
+    "headline_bf16_T16384_D128": {"fwd": 1.765e9, "delta": 5.411e8, "dq": 2.122e9, "dkdv": 1.752e9},
 }
 
 
