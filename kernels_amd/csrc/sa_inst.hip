@@ -22,14 +22,29 @@ using ElemT = __bf16;
 #error "SA_DTYPE_ID must be 0, 1 or 2"
 #endif
 
-template <typename K> static int prepare(K kernel, size_t lds_bytes, std::once_flag& once) {
-  int rc = 0;
-  std::call_once(once, [&] {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    rc = (int)e;
-  });
-  return rc;
+// Kernels whose dynamic LDS exceeds the 64 KiB default need the limit raised once per kernel
+// and per device (the attribute belongs to the device that is current when it is set).  The
+// outcome of that one call is kept and handed to every caller on that device.
+struct PrepareState {
+  static constexpr int kMaxDevices = 64;
+  std::mutex mu;
+  bool done[kMaxDevices] = {};
+  int rc[kMaxDevices] = {};
+};
+template <typename K> static int prepare(K kernel, size_t lds_bytes, PrepareState& state) {
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= PrepareState::kMaxDevices) {
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+  }
+  std::lock_guard<std::mutex> lock(state.mu);
+  if (!state.done[dev]) {
+    state.rc[dev] = (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    state.done[dev] = true;
+  }
+  return state.rc[dev];
 }
 
 static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -62,7 +77,7 @@ template <int D, int NW> static int fwd2_launch(FwdParams p, hipStream_t st) {
   constexpr size_t patches = (size_t)NW * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
   constexpr size_t lds = stages > patches ? stages : patches;
   auto kern = fwd2_kernel<ElemT, D, C::FWD2_QB, NW, C::FWD_TK, C::FWD2_NST>;
-  static std::once_flag once;
+  static PrepareState once;
   if (int rc = prepare(kern, lds, once)) return rc;
   p.n_tiles = (int)ceil_div(p.T, TQ);
   const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
@@ -78,7 +93,7 @@ template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
     constexpr int TQ = C::NW * 32;
     constexpr size_t lds = (size_t)2 * 2 * C::FWD_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
     auto kern = fwd_kernel<ElemT, D, C::NW, C::FWD_TK>;
-    static std::once_flag once;
+    static PrepareState once;
     if (int rc = prepare(kern, lds, once)) return rc;
     p.n_tiles = (int)ceil_div(p.T, TQ);
     const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
@@ -113,7 +128,7 @@ template <int D, int NW> static int dq2_launch(BwdParams p, hipStream_t st) {
   constexpr size_t patches = (size_t)NW * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
   constexpr size_t lds = stages > patches ? stages : patches;
   auto kern = dq2_kernel<ElemT, D, NW, C::DQ2_TK, C::DQ2_NST>;
-  static std::once_flag once;
+  static PrepareState once;
   if (int rc = prepare(kern, lds, once)) return rc;
   p.n_tiles = (int)ceil_div(p.T, TQ);
   const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
@@ -129,7 +144,7 @@ template <int D> static int dq_d(BwdParams p, hipStream_t st) {
     constexpr int TQ = C::NW * 32;
     constexpr size_t lds = (size_t)2 * 2 * C::DQ_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
     auto kern = dq_kernel<ElemT, D, C::NW, C::DQ_TK>;
-    static std::once_flag once;
+    static PrepareState once;
     if (int rc = prepare(kern, lds, once)) return rc;
     p.n_tiles = (int)ceil_div(p.T, TQ);
     const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
@@ -153,7 +168,7 @@ template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
     constexpr size_t patches = (size_t)C::DKDV2_NW * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
     constexpr size_t lds = stages > patches ? stages : patches;
     auto kern = dkdv2_kernel<ElemT, D, C::DKDV2_NW, C::DKDV2_TQ, C::DKDV2_NST>;
-    static std::once_flag once;
+    static PrepareState once;
     if (int rc = prepare(kern, lds, once)) return rc;
     p.n_tiles = (int)ceil_div(p.T, TKB);
     const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
@@ -165,7 +180,7 @@ template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
     constexpr size_t lds =
         (size_t)2 * (2 * C::DKDV_TQ * TileGeom<ElemT, D>::PITCH * sizeof(ElemT) + 2 * C::DKDV_TQ * sizeof(float));
     auto kern = dkdv_kernel<ElemT, D, C::NW, C::DKDV_TQ>;
-    static std::once_flag once;
+    static PrepareState once;
     if (int rc = prepare(kern, lds, once)) return rc;
     p.n_tiles = (int)ceil_div(p.T, TKB);
     const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;

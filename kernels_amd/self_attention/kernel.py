@@ -13,7 +13,7 @@ import torch
 import torch.nn.functional as F
 
 from streaming_attention import _lib
-from streaming_attention.ops import _dtype_id, _kernel_layout, _lens_args, _stream
+from streaming_attention.ops import _dtype_id, _kernel_layout, _lens_args, _stream, _validate_placement
 
 _HEAD_DIMS = (16, 32, 64, 128, 256)
 
@@ -28,6 +28,7 @@ def attention_forward_adapter(
     autotune: bool,
     prescale: bool,
 ) -> torch.Tensor:
+    _validate_placement(q, k, v, lens)
     batch, heads, T, head_dim = q.shape
     # same conditions as src/self_attention/kernel.py:372-379
     assert head_dim in _HEAD_DIMS

@@ -52,8 +52,22 @@ def _stream(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def _validate(q, k, v, lens, context_size, back_contexts, sm_scale):
+def _validate_placement(q, k, v, lens, *others):
+    """The kernels index k, v (and o, dO) with q's batch and head counts and dereference every
+    pointer on q's device, so a tensor that lives elsewhere or has fewer batches / heads (an
+    un-expanded grouped-query k or v) must be refused before any ``data_ptr()`` is taken."""
+    assert q.ndim == 4 and k.ndim == 4 and v.ndim == 4
+    assert k.shape[:2] == q.shape[:2] and v.shape[:2] == q.shape[:2], "k and v need q's batch and head sizes"
+    assert k.device == q.device and v.device == q.device, "q, k and v must be on one device"
+    assert lens is None or lens.device == q.device, "lens must be on the device of q"
+    for t in others:
+        assert t.shape == q.shape, "o and dO need q's shape"
+        assert t.device == q.device, "o and dO must be on the device of q"
+
+
+def _validate(q, k, v, lens, context_size, back_contexts, sm_scale, *others):
     # same conditions, same exception type as kernel.py:1288-1295
+    _validate_placement(q, k, v, lens, *others)
     batch, _, T, head_dim = q.shape
     assert back_contexts >= 0 and context_size >= 1
     assert head_dim in _HEAD_DIMS
@@ -131,7 +145,7 @@ def attention_backward_adapter(
     prescale_qk: bool,
     precision: str,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    _validate(q, k, v, lens, context_size, back_contexts, sm_scale)
+    _validate(q, k, v, lens, context_size, back_contexts, sm_scale, o, do)
     B, H, T, D = q.shape
     lib = _lib.load()
     DQ = torch.empty(q.shape, dtype=q.dtype, device=q.device)
