@@ -43,6 +43,10 @@ extern "C" {
 #define SA_ERR_ARG (-3)
 #define SA_ERR_LAYOUT (-4)
 #define SA_ERR_TOO_LARGE (-5)
+#define SA_ERR_SCRATCH (-6)
+
+/* Rows (B*H*T) that the static workspace of sa_backward_static holds: 8 MiB of float32 per GPU. */
+#define SA_STATIC_MAX_ROWS (1 << 21)
 
 /* Forward pass: O = softmax_window(sm_scale * Q K^T) V, LSE = log2 sum exp (scaled scores).
  * Replaces the launch of `_streaming_attn_fwd` inside `attention_forward_adapter`
@@ -100,6 +104,26 @@ int sa_backward(const void* q, const void* k, const void* v,
                 int context_size, int back_contexts, float sm_scale,
                 int dtype, void* stream);
 
+/* sa_backward for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the same three kernels, with the
+ * [B,H,T] float32 row-sum workspace taken from a static device array inside the library instead
+ * of a `delta` argument.  It has no counterpart in the reference.
+ *   - B*H*T must not exceed SA_STATIC_MAX_ROWS (sa_query(10)); larger problems return
+ *     SA_ERR_SCRATCH and launch nothing.
+ *   - Calls nothing that allocates or frees.  The first call on a device looks the array's
+ *     address up (hipGetSymbolAddress); make that call outside a graph capture.
+ *   - Every call on one GPU uses that GPU's single array: calls that overlap on one GPU (two
+ *     streams, two threads) race.  Calls on one stream are ordered and safe. */
+int sa_backward_static(const void* q, const void* k, const void* v,
+                       const int32_t* lens, int64_t lens_stride,
+                       const void* o, const void* d_o, const float* lse,
+                       void* dq, void* dk, void* dv,
+                       const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                       const int64_t* o_strides, const int64_t* do_strides,
+                       int B, int H, int T, int D,
+                       int context_size, int back_contexts, float sm_scale,
+                       int dtype, void* stream);
+
 /* Static facts about the build, answerable without a GPU.  Replaces the reference's
  * launch-configuration tables (src/streaming_attention/kernel.py:17-85, 1143-1267) as the
  * place where tile shapes are looked up.
@@ -111,6 +135,7 @@ int sa_backward(const void* q, const void* k, const void* v,
  *          7, 8: waves per workgroup of the wide / narrow forward and dQ kernels used for the
  *                16-bit types at D in {64, 128} (each wave owns 32 queries)
  *          9: smallest context_size for which the wide kernels are chosen
+ *         10: rows (B*H*T) the static workspace of sa_backward_static holds
  *   anything else: -1 */
 int sa_query(int what);
 

@@ -1,9 +1,15 @@
 // extern "C" surface of libstreaming_attention.so: argument checks, parameter packing
 // and dispatch on the element type.  See include/streaming_attention.h for the contract.
+#include <mutex>
 #include "../../include/streaming_attention.h"
 #include "sa_launch.h"
 
 using namespace sa;
+
+// Workspace of sa_backward_static: the [B,H,T] float32 row sums that sa_backward takes from its
+// caller.  One copy per GPU, held until the process ends.  In host code this name only stands
+// for the symbol; the memory is reached through the address hipGetSymbolAddress returns.
+static __device__ __align__(256) float sa_static_delta[SA_STATIC_MAX_ROWS];
 
 namespace {
 
@@ -162,6 +168,40 @@ int sa_backward(const void* q, const void* k, const void* v, const int32_t* lens
                    back_contexts, sm_scale, dtype, stream);
 }
 
+int sa_backward_static(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
+                       const void* o, const void* d_o, const float* lse, void* dq, void* dk, void* dv,
+                       const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
+                       const int64_t* gs, int B, int H, int T, int D, int context_size, int back_contexts,
+                       float sm_scale, int dtype, void* stream) {
+  if (int rc = check_common(B, H, T, D, dtype)) return rc;
+  if ((int64_t)B * H * T > (int64_t)SA_STATIC_MAX_ROWS) return SA_ERR_SCRATCH;
+  // each device has its own copy of the array at its own address: look it up once per device
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static float* base[kMaxDevices] = {};
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return SA_ERR_ARG;
+  float* delta = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (!base[dev]) {
+      void* ptr = nullptr;
+      if (hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(sa_static_delta)); e != hipSuccess) return (int)e;
+      base[dev] = static_cast<float*>(ptr);
+    }
+    delta = base[dev];
+  }
+  if (!delta) return SA_ERR_ARG;
+  // every row the kernels read is written by the delta pass first: nothing to clear
+  if (int rc = sa_bwd_delta(o, d_o, delta, os, gs, B, H, T, D, dtype, stream)) return rc;
+  if (int rc = sa_bwd_dkdv(q, k, v, lens, lens_stride, d_o, lse, delta, dk, dv, qs, ks, vs, gs, B, H, T, D,
+                           context_size, back_contexts, sm_scale, dtype, stream))
+    return rc;
+  return sa_bwd_dq(q, k, v, lens, lens_stride, d_o, lse, delta, dq, qs, ks, vs, gs, B, H, T, D, context_size,
+                   back_contexts, sm_scale, dtype, stream);
+}
+
 int sa_query(int what) {
   switch (what) {
     case 0: return 1;
@@ -174,6 +214,7 @@ int sa_query(int what) {
     case 7: return Cfg<__bf16>::WIDE_NW;
     case 8: return Cfg<__bf16>::NARROW_NW;
     case 9: return Cfg<__bf16>::WIDE_CHUNK;
+    case 10: return SA_STATIC_MAX_ROWS;
   }
   return -1;
 }
@@ -186,6 +227,7 @@ const char* sa_error_string(int code) {
     case SA_ERR_ARG: return "invalid argument (null pointer, negative size, context_size < 1 or back_contexts < 0)";
     case SA_ERR_LAYOUT: return "unsupported layout (dim stride must be 1; pointers and strides 16-byte aligned)";
     case SA_ERR_TOO_LARGE: return "problem too large for one launch";
+    case SA_ERR_SCRATCH: return "B*H*T exceeds the static workspace of sa_backward_static (see sa_query(10))";
   }
   return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
 }

@@ -30,6 +30,9 @@ SIGNATURES = {
     "sa_backward": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                     _pi64, _pi64, _pi64, _pi64, _pi64,
                     _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp],
+    "sa_backward_static": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp,
+                           _pi64, _pi64, _pi64, _pi64, _pi64,
+                           _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp],
     "sa_query": [_i32],
     "sa_error_string": [_i32],
 }

@@ -29,7 +29,7 @@ def _declared_symbols():
 
 def test_header_symbols_exported(lib):
     names = _declared_symbols()
-    assert names == ["sa_backward", "sa_bwd_delta", "sa_bwd_dkdv", "sa_bwd_dq", "sa_error_string",
+    assert names == ["sa_backward", "sa_backward_static", "sa_bwd_delta", "sa_bwd_dkdv", "sa_bwd_dq", "sa_error_string",
                      "sa_forward", "sa_query"]
     for n in names:
         assert getattr(lib, n) is not None
@@ -45,7 +45,8 @@ def test_query_and_error_strings(lib):
     assert (lib.sa_query(7), lib.sa_query(8)) == (8, 4) and lib.sa_query(9) == 256
     assert lib.sa_query(99) == -1
     assert b"success" in lib.sa_error_string(0)
-    for code in (-1, -2, -3, -4, -5):
+    assert lib.sa_query(10) == 1 << 21
+    for code in (-1, -2, -3, -4, -5, -6):
         assert len(lib.sa_error_string(code)) > 10
 
 
@@ -73,6 +74,9 @@ def test_validation_codes_without_gpu(lib):
     assert fwd(T=2**22, qs=(ctypes.c_int64 * 4)(2**33, 64, 2048, 1)) == -5   # row offsets beyond 32 bits
     assert fwd(B=0) == 0 and fwd(T=0) == 0                         # empty problems are no-ops
     assert lib.sa_bwd_delta(p, p, None, st, st, 1, 1, 8, 64, 2, None) == -3
+    # the static-workspace backward refuses what its array cannot hold, before any HIP call
+    assert lib.sa_backward_static(p, p, p, None, 0, p, p, p, p, p, p, st, st, st, st, st,
+                                  1, 33, 2**16, 64, 4, 1, 0.125, 2, None) == -6
     assert lib.sa_bwd_delta(p, p, p, st, st, 1, 1, 8, 17, 2, None) == -2
 
 
@@ -147,6 +151,33 @@ def test_validation_asserts_like_reference():
         ops._validate(q, q, q, lens.long(), 4, 1, 0.1)                          # lens dtype
     with pytest.raises(AssertionError):
         ops._validate(q, q, q, lens[:1], 4, 1, 0.1)                             # lens length
+
+
+def test_placement_validation_launches_nothing():
+    """A tensor on another device, or k / v with fewer batches or heads than q (an un-expanded
+    grouped-query tensor), is refused with an AssertionError before any pointer is taken."""
+    from streaming_attention import ops
+
+    q = torch.zeros(2, 4, 8, 64)
+    lens = torch.tensor([8, 8], dtype=torch.int32)
+    meta = torch.zeros(2, 4, 8, 64, device="meta")
+    with pytest.raises(AssertionError):
+        ops._validate(q, meta, q, lens, 4, 1, 0.1)                              # k elsewhere
+    with pytest.raises(AssertionError):
+        ops._validate(q, q, meta, lens, 4, 1, 0.1)                              # v elsewhere
+    with pytest.raises(AssertionError):
+        ops._validate(q, q, q, lens.to("meta"), 4, 1, 0.1)                      # lens elsewhere
+    with pytest.raises(AssertionError):
+        ops._validate(q, torch.zeros(2, 1, 8, 64), q, lens, 4, 1, 0.1)          # k with one head
+    with pytest.raises(AssertionError):
+        ops._validate(q, q, torch.zeros(1, 4, 8, 64), lens, 4, 1, 0.1)          # v with one batch
+    with pytest.raises(AssertionError):
+        ops._validate(q, q, q, lens, 4, 1, 0.1, meta, q)                        # o elsewhere
+    with pytest.raises(AssertionError):
+        ops._validate(q, q, q, lens, 4, 1, 0.1, q, torch.zeros(2, 4, 9, 64))    # dO of another shape
+    ops._validate(q, q, q, lens, 4, 1, 0.1, q, q)
+    with pytest.raises(AssertionError):
+        ops._validate_placement(q, q[:, :1], q, None)
 
 
 def test_kernel_layout_rule():
