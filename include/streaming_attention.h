@@ -136,6 +136,8 @@ int sa_backward_static(const void* q, const void* k, const void* v,
  *                16-bit types at D in {64, 128} (each wave owns 32 queries)
  *          9: smallest context_size for which the wide kernels are chosen
  *         10: rows (B*H*T) the static workspace of sa_backward_static holds
+ *         11: smallest context_size for which the software-pipelined dK/dV kernel is chosen
+ *             (16-bit types, D in {64, 128})
  *   anything else: -1 */
 int sa_query(int what);
 

@@ -215,6 +215,7 @@ int sa_query(int what) {
     case 8: return Cfg<__bf16>::NARROW_NW;
     case 9: return Cfg<__bf16>::WIDE_CHUNK;
     case 10: return SA_STATIC_MAX_ROWS;
+    case 11: return Cfg<__bf16>::DKDV3_MIN_CHUNK;
   }
   return -1;
 }

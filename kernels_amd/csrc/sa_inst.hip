@@ -8,6 +8,7 @@
 #include "sa_fwd.h"
 #else
 #include "sa_bwd.h"
+#include "sa_bwd3.h"
 #endif
 
 namespace sa {
@@ -159,9 +160,33 @@ template <> int launch_dq<ElemT, SA_DGROUP>(const BwdParams& p, int D, hipStream
 #undef X
 }
 #else
+template <int D> static int dkdv3_launch(BwdParams p, hipStream_t st) {
+  using C = Cfg<ElemT>;
+  if constexpr (C::fwd2(D)) {
+    constexpr int TKB = 128, TQ = 64;
+    // tile stages; the epilogue's row patches (one per wave) reuse the same memory
+    constexpr size_t stages = (size_t)C::DKDV3_NST * (2 * TQ * D * sizeof(ElemT) + 2 * TQ * sizeof(float));
+    constexpr size_t patches = (size_t)4 * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
+    constexpr size_t lds = stages > patches ? stages : patches;
+    auto kern = dkdv3_kernel<ElemT, D, C::DKDV3_NST>;
+    static PrepareState once;
+    if (int rc = prepare(kern, lds, once)) return rc;
+    p.n_tiles = (int)ceil_div(p.T, TKB);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, st, p);
+    return (int)hipGetLastError();
+  } else {
+    return SA_ERR_HEAD_DIM;
+  }
+}
 template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
+    // The pipelined kernel makes every wave walk the whole window of its workgroup's 128 keys;
+    // that wastes nothing once a chunk holds at least those 128 keys.  Smaller chunks go to the
+    // kernel whose waves skip the query tiles outside their own 32 keys' windows.
+    if (C::pipelined_dkdv(p.C)) return dkdv3_launch<D>(p, st);
     constexpr int TKB = C::DKDV2_NW * 32;
     constexpr size_t stages =
         (size_t)C::DKDV2_NST * (2 * C::DKDV2_TQ * D * sizeof(ElemT) + 2 * C::DKDV2_TQ * sizeof(float));

@@ -33,6 +33,12 @@ template <typename T, int DGROUP> int launch_dkdv(const BwdParams& p, int D, hip
 #ifndef SA_DKDV2_NST
 #define SA_DKDV2_NST 2
 #endif
+#ifndef SA_DKDV3_MIN_CHUNK
+#define SA_DKDV3_MIN_CHUNK 128
+#endif
+#ifndef SA_DKDV3_NST
+#define SA_DKDV3_NST 3
+#endif
 #ifndef SA_FWD2_NST
 #define SA_FWD2_NST 2
 #endif
@@ -48,6 +54,10 @@ template <typename T> struct Cfg {
   static constexpr bool wide(int chunk) { return chunk >= WIDE_CHUNK; }
   static constexpr int DQ2_TK = SA_DQ2_TK, DQ2_NST = SA_DQ2_NST;
   static constexpr int DKDV2_NW = SA_DKDV2_NW, DKDV2_TQ = SA_DKDV2_TQ, DKDV2_NST = SA_DKDV2_NST;
+  // smallest chunk for which the software-pipelined dK/dV kernel is chosen (0x7fffffff: never)
+  static constexpr int DKDV3_MIN_CHUNK = SA_DKDV3_MIN_CHUNK;
+  static constexpr bool pipelined_dkdv(int chunk) { return chunk >= DKDV3_MIN_CHUNK; }
+  static constexpr int DKDV3_NST = SA_DKDV3_NST;
   static constexpr int FWD2_QB = SA_FWD2_QB;
   static constexpr int FWD2_NST = SA_FWD2_NST;
 #ifdef SA_FWD2_DISABLE

@@ -46,6 +46,7 @@ def test_query_and_error_strings(lib):
     assert lib.sa_query(99) == -1
     assert b"success" in lib.sa_error_string(0)
     assert lib.sa_query(10) == 1 << 21
+    assert lib.sa_query(11) == 128
     for code in (-1, -2, -3, -4, -5, -6):
         assert len(lib.sa_error_string(code)) > 10
 
