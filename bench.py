@@ -7,8 +7,15 @@ B=4, H=16, T=16384, D=128, bf16, chunk 256, 8 back chunks, lens ~ U{T/2..T}.
 
 Prints one JSON line:
   value      effective TFLOP/s = 14*D*H*P / step time, P = unmasked (query, key) pairs
-  roofline   the dominant kernel (longest average launch) timed on its own with HIP events
-             on the launch stream, against the dense bf16 MFMA peak
+             (value_block_granular counts whole chunk x chunk blocks that hold any allowed pair)
+  roofline   the dominant kernel (longest average launch) timed on its own with HIP events on the
+             launch stream.  The bound is chosen per workload from the step's arithmetic intensity
+             (algorithmic flop / algorithmic HBM bytes against the machine balance): matrix-pipe
+             bound workloads report TFLOP/s against the MFMA peak of their element type, HBM-bound
+             ones GB/s against 8 TB/s.  `traffic` (HBM bytes per launch) comes from rocprofv3
+             counter runs of this script, quoted from the committed summaries under profiles/.
+  measured_ceilings  what a bare MFMA stream (constant and random bf16 operands) and a plain copy
+             reach on this GPU in this run (libsa_probe.so), beside the published peaks
   cpu_baseline  the CPU oracle forward+backward in fp32 on the host cores, on a bounded sample
              of the same workload (one batch element, all heads), and the reference's dense-mask
              SDPA formulation on the reference's CPU-sized configuration
@@ -26,7 +33,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "kernels_amd"))
 sys.path.insert(0, ROOT)
 
-PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 / fp16 MFMA, published
+PEAK_F32_TFLOPS = 157.3     # MI355X dense fp32 MFMA, published
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
 
 WORKLOADS = {
@@ -51,6 +59,18 @@ def unmasked_pairs(T, C, R, lens_list):
             keys = min((c + 1) * C, L) - max(0, c - R) * C
             total += rows * keys
             c += 1
+    return total
+
+
+def unmasked_block_pairs(T, C, R, lens_list):
+    """Pairs in chunk x chunk blocks that hold at least one allowed pair (the figure a
+    block-skipping kernel cannot go below), per head, summed over the batch."""
+    total = 0
+    for L in lens_list:
+        L = min(int(L), T)
+        n = -(-L // C)                      # chunks that hold a valid position
+        for c in range(n):
+            total += C * C * (min(c, R) + 1)
     return total
 
 
@@ -180,11 +200,35 @@ def cpu_baseline(w, name, budget_s=12.0):
 
 
 # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (separate --pmc runs of this script, scaled by
-# what the same counters read for the 1 GiB copy of --calibrate-copy: x2.000 and x1.000).  Counter runs
-# cannot be made from inside a timed run, so the figures of the committed profile summary are quoted here.
+# what the same counters read for the 1 GiB copy of --calibrate-copy).  Counter runs cannot be made from
+# inside a timed run, so the figures of the committed summaries under profiles/ are quoted here; a
+# workload or kernel without a committed counter run reports null.
 HBM_BYTES_PER_LAUNCH = {
     "headline_bf16_T16384_D128": {"fwd": 1.765e9, "delta": 5.411e8, "dq": 2.122e9, "dkdv": 1.752e9},
 }
+TRAFFIC_SOURCE = "quoted from the rocprofv3 FETCH_SIZE/WRITE_SIZE summary under profiles/ (not measured in this run)"
+
+
+def measured_ceilings():
+    """Bare MFMA stream and plain copy on this GPU, through libsa_probe.so (bench support code)."""
+    import ctypes
+
+    path = os.path.join(ROOT, "kernels_amd", "streaming_attention", "libsa_probe.so")
+    if not os.path.exists(path):
+        return {"error": f"{path} not built (make -C kernels_amd/csrc)"}
+    lib = ctypes.CDLL(path)
+    lib.sa_probe_mfma_bf16.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    lib.sa_probe_copy.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    out = {}
+    v = ctypes.c_double()
+    for name, rnd in (("bf16_mfma_constant_operands_tflops", 0), ("bf16_mfma_random_operands_tflops", 1)):
+        rc = lib.sa_probe_mfma_bf16(rnd, 4000, 2, ctypes.byref(v))
+        out[name] = v.value if rc == 0 else f"hip error {rc}"
+    rc = lib.sa_probe_copy(1 << 30, 5, ctypes.byref(v))
+    out["copy_read_plus_write_gbs"] = v.value if rc == 0 else f"hip error {rc}"
+    out["note"] = ("v_mfma_f32_32x32x16_bf16 only, 2 waves per SIMD, 8 accumulator chains per wave; copy of 1 GiB "
+                   "with 16-byte accesses, bytes read + bytes written")
+    return out
 
 
 def reference_sweep(device, iters=20):
@@ -243,6 +287,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-ceilings", action="store_true", help="skip the MFMA / copy ceiling measurement")
     ap.add_argument("--kernel-iters", type=int, default=10)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy (known traffic) for scaling HBM counters")
@@ -293,31 +338,67 @@ def main():
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     value = flops_step / (ms_per_step * 1e-3) / 1e12
 
+    # the same steps once more, each bracketed by events on the stream they run on, for the median
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for e0, e1 in evs:
+        e0.record()
+        step()
+        e1.record()
+    torch.cuda.synchronize()
+    per_step = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+    median_ms = per_step[len(per_step) // 2] if len(per_step) % 2 else \
+        0.5 * (per_step[len(per_step) // 2 - 1] + per_step[len(per_step) // 2])
+
     kt = time_kernels(w, args.kernel_iters)
     # GEMMs each kernel performs per unmasked pair: fwd S,PV; dq S,dP,dQ; dkdv S,dP,dV,dK
     kernel_flops = {"fwd": 4.0 * D * H * P, "dq": 6.0 * D * H * P, "dkdv": 8.0 * D * H * P}
-    dom = max(kernel_flops, key=lambda n: kt[n])
-    achieved = kernel_flops[dom] / (kt[dom] * 1e-3) / 1e12
     es = 4 if w["dtype"] == "float32" else 2
     N = B * H * T
+    tensor = float(N) * D * es
+    # algorithmic HBM bytes per launch: every operand read once, every result written once
+    kernel_bytes = {"fwd": 4.0 * tensor + 4.0 * N, "delta": 2.0 * tensor + 4.0 * N,
+                    "dq": 5.0 * tensor + 8.0 * N, "dkdv": 6.0 * tensor + 8.0 * N}
+    step_bytes = 12.0 * tensor + 16.0 * N
+    peak_tflops = PEAK_F32_TFLOPS if w["dtype"] == "float32" else PEAK_BF16_TFLOPS
+    balance = peak_tflops * 1e12 / (PEAK_HBM_GBS * 1e9)            # flop per byte at which the two roofs meet
+    intensity = flops_step / step_bytes
+    bound = "mfma" if intensity >= balance else "hbm"
+    dom = max(kernel_flops, key=lambda n: kt[n])
+    traffic = HBM_BYTES_PER_LAUNCH.get(args.workload, {}).get(dom)
+    if bound == "mfma":
+        achieved = kernel_flops[dom] / (kt[dom] * 1e-3) / 1e12
+        roofline = {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": peak_tflops, "unit": "TFLOP/s",
+                    "frac": achieved / peak_tflops}
+    else:
+        achieved = kernel_bytes[dom] / (kt[dom] * 1e-3) / 1e9
+        roofline = {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": achieved / PEAK_HBM_GBS}
+    roofline.update({"traffic": traffic, "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
+                     "algorithmic_bytes": kernel_bytes[dom], "algorithmic_flops": kernel_flops[dom],
+                     "arithmetic_intensity_flop_per_byte": intensity, "machine_balance_flop_per_byte": balance})
+    P_blocks = unmasked_block_pairs(T, C, R, w["lens_list"])
     result = {
         "metric": "effective TFLOP/s fwd+bwd (unmasked blocks) at 1 GPU; % of bf16 MFMA peak",
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": ms_per_step, "median_ms": median_ms, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None,
         "dtype": {"bfloat16": "bf16", "float16": "f16", "float32": "f32"}[w["dtype"]],
         "data": "synthetic, all zeros (diagnostic run)" if args.zero_inputs else "synthetic",
         "config": {"workload": args.workload, "B": B, "H": H, "T": T, "D": D, "context_size": C,
                    "back_contexts": R, "lens": w["lens_list"], "unmasked_pairs_per_head": P,
-                   "flops_per_step": flops_step},
+                   "flops_per_step": flops_step, "algorithmic_bytes_per_step": step_bytes},
         "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
-        "peaks_used": {"bf16_mfma_tflops": PEAK_BF16_TFLOPS, "hbm_gbs": PEAK_HBM_GBS},
+        "value_block_granular": 14.0 * D * H * P_blocks / (ms_per_step * 1e-3) / 1e12,
+        "step_hbm_gbs": step_bytes / (ms_per_step * 1e-3) / 1e9,
+        "peaks_used": {"bf16_mfma_tflops": PEAK_BF16_TFLOPS, "f32_mfma_tflops": PEAK_F32_TFLOPS,
+                       "hbm_gbs": PEAK_HBM_GBS},
         "kernel_ms": kt,
         "kernel_tflops": {n: kernel_flops[n] / (kt[n] * 1e-3) / 1e12 for n in kernel_flops},
-        "delta_gbs": (2.0 * N * D * es + 4.0 * N) / (kt["delta"] * 1e-3) / 1e9,
-        "roofline": {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
-                     "traffic": HBM_BYTES_PER_LAUNCH.get(args.workload, {}).get(dom)},
+        "kernel_gbs": {n: kernel_bytes[n] / (kt[n] * 1e-3) / 1e9 for n in kernel_bytes},
+        "roofline": roofline,
     }
+    if not args.no_ceilings:
+        result["measured_ceilings"] = measured_ceilings()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, args.workload)
     print(json.dumps(result))
