@@ -8,7 +8,7 @@ work of the previous 32-query block.  The compiler's register allocator does not
 files), so the loop is emitted here with every register chosen by hand, every s_waitcnt counted,
 and the hazards the hardware leaves to software spaced out by construction.
 
-Register map (D = 128; D = 64 uses the lower half of the per-D groups):
+Register map (the kernel is built for D = 128):
   a[0:63]    dV^T blocks (16 registers per 32 columns of D)     a[64:127]  dK^T blocks
   a[128:159] K fragments (4 registers per 16 columns of D)      a[160:191] V fragments (negated)
   v[0:31]    score accumulators of the even / odd block         v[32:63]   delta - dP accumulators
@@ -423,7 +423,7 @@ def main():
     print("#define SA_DKDV3_NUM_SCALARS %d" % len(SCALARS))
     for i, nm in enumerate(SCALARS):
         print(f"#define SA_DKDV3_SC_{nm.upper()} {i}")
-    for D in (64, 128):
+    for D in (128,):
         for dt in ("bf16", "f16"):
             print(generate(D, dt))
 

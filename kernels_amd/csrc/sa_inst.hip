@@ -162,7 +162,7 @@ template <> int launch_dq<ElemT, SA_DGROUP>(const BwdParams& p, int D, hipStream
 #else
 template <int D> static int dkdv3_launch(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
-  if constexpr (C::fwd2(D)) {
+  if constexpr (C::fwd2(D) && D == 128) {
     constexpr int TKB = 128, TQ = 64;
     // tile stages; the epilogue's row patches (one per wave) reuse the same memory
     constexpr size_t stages = (size_t)C::DKDV3_NST * (2 * TQ * D * sizeof(ElemT) + 2 * TQ * sizeof(float));
@@ -183,10 +183,12 @@ template <int D> static int dkdv3_launch(BwdParams p, hipStream_t st) {
 template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
-    // The pipelined kernel makes every wave walk the whole window of its workgroup's 128 keys;
-    // that wastes nothing once a chunk holds at least those 128 keys.  Smaller chunks go to the
-    // kernel whose waves skip the query tiles outside their own 32 keys' windows.
-    if (C::pipelined_dkdv(p.C)) return dkdv3_launch<D>(p, st);
+    // The pipelined kernel (head dimension 128) makes every wave walk the whole window of its
+    // workgroup's 128 keys; that wastes nothing once a chunk holds at least those 128 keys.  Smaller
+    // chunks go to the kernel whose waves skip the query tiles outside their own 32 keys' windows.
+    if constexpr (D == 128) {
+      if (C::pipelined_dkdv(p.C, D)) return dkdv3_launch<D>(p, st);
+    }
     constexpr int TKB = C::DKDV2_NW * 32;
     constexpr size_t stages =
         (size_t)C::DKDV2_NST * (2 * C::DKDV2_TQ * D * sizeof(ElemT) + 2 * C::DKDV2_TQ * sizeof(float));

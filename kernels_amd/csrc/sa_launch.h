@@ -56,7 +56,10 @@ template <typename T> struct Cfg {
   static constexpr int DKDV2_NW = SA_DKDV2_NW, DKDV2_TQ = SA_DKDV2_TQ, DKDV2_NST = SA_DKDV2_NST;
   // smallest chunk for which the software-pipelined dK/dV kernel is chosen (0x7fffffff: never)
   static constexpr int DKDV3_MIN_CHUNK = SA_DKDV3_MIN_CHUNK;
-  static constexpr bool pipelined_dkdv(int chunk) { return chunk >= DKDV3_MIN_CHUNK; }
+  // ... and only at head dimension 128: at 64 a block step has half the MFMAs for the same softmax
+  // arithmetic, the loop is bound by its vector work and dkdv2 is faster (0.23 against 0.30 ms at
+  // B=8, H=16, T=4096, chunk 128)
+  static constexpr bool pipelined_dkdv(int chunk, int D) { return D == 128 && chunk >= DKDV3_MIN_CHUNK; }
   static constexpr int DKDV3_NST = SA_DKDV3_NST;
   static constexpr int FWD2_QB = SA_FWD2_QB;
   static constexpr int FWD2_NST = SA_FWD2_NST;

@@ -13,7 +13,7 @@ import torch
 import torch.nn.functional as F
 
 from streaming_attention import _lib
-from streaming_attention.ops import _dtype_id, _kernel_layout, _lens_args, _stream, _validate_placement
+from streaming_attention.ops import _dtype_id, _kernel_layout, _lens_args, _on_device, _stream, _validate_placement
 
 _HEAD_DIMS = (16, 32, 64, 128, 256)
 
@@ -44,7 +44,7 @@ def attention_forward_adapter(
         return O
     qk, kk, vk = _kernel_layout(q), _kernel_layout(k), _kernel_layout(v)
     lens_ptr, lens_stride = _lens_args(lens)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         rc = lib.sa_forward(
             qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), lens_ptr, lens_stride, O.data_ptr(), None,
             _lib.strides4(qk), _lib.strides4(kk), _lib.strides4(vk),

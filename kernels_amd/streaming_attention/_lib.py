@@ -75,5 +75,16 @@ def check(rc: int, what: str) -> None:
         raise RuntimeError(f"{what} failed with code {rc}: {msg}")
 
 
+_stride_cache: dict = {}
+
+
 def strides4(t) -> ctypes.Array:
-    return (ctypes.c_int64 * 4)(*t.stride())
+    """The four element strides of ``t`` as an int64[4]; arrays are cached per stride tuple (the
+    library only reads them)."""
+    key = t.stride()
+    arr = _stride_cache.get(key)
+    if arr is None:
+        if len(_stride_cache) > 4096:
+            _stride_cache.clear()
+        arr = _stride_cache[key] = (ctypes.c_int64 * 4)(*key)
+    return arr

@@ -32,6 +32,9 @@ def _kernel_layout(t: torch.Tensor) -> torch.Tensor:
     contiguous copy.  The kernels address the rows of one (batch, head) slice with 32-bit
     byte offsets (a contiguous tensor is within that range up to tens of millions of positions)."""
     es = t.element_size()
+    if t.is_contiguous() and t.data_ptr() % _VEC_BYTES == 0 and t.shape[-1] * es % _VEC_BYTES == 0 \
+            and (t.shape[-2] + 1024) * t.shape[-1] * es < 2**32:
+        return t          # the common case, without looking at every stride
     vec = _VEC_BYTES // es
     ok = (
         t.stride(-1) == 1
@@ -50,6 +53,26 @@ def _lens_args(lens: Optional[torch.Tensor]):
 
 def _stream(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _on_device:
+    """``torch.cuda.device(dev)`` that does nothing when ``dev`` is already current: entering the
+    real context costs more than the launch of a small kernel."""
+
+    __slots__ = ("ctx",)
+
+    def __init__(self, device):
+        idx = device.index
+        self.ctx = None if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
 
 
 def _validate_placement(q, k, v, lens, *others):
@@ -103,7 +126,7 @@ def attention_forward_adapter(
     if q.numel() > 0:
         qk, kk, vk = _kernel_layout(q), _kernel_layout(k), _kernel_layout(v)
         lens_ptr, lens_stride = _lens_args(lens)
-        with torch.cuda.device(q.device):
+        with _on_device(q.device):
             rc = lib.sa_forward(
                 qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), lens_ptr, lens_stride,
                 O.data_ptr(), LSE.data_ptr() if LSE is not None else None,
@@ -162,7 +185,7 @@ def attention_backward_adapter(
     dt = _dtype_id(q.dtype)
     C = min(int(context_size), 2**31 - 1)
     R = min(int(back_contexts), 2**31 - 1)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         stream = _stream(q.device)
         if lse.numel() != B * H * T or lse.device != q.device:
             # forward was run with return_lse=False: rebuild the log-sum-exp

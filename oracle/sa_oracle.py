@@ -75,9 +75,20 @@ def unmasked_pairs(T: int, context_size: int, back_contexts: int, L) -> int:
     return total
 
 
-def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=None):
+def _round_like(x, dtype):
+    """float64 array -> rounded to ``dtype`` (torch) -> float64."""
+    return torch.from_numpy(np.ascontiguousarray(x)).to(dtype).double().numpy()
+
+
+def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=None, round_dtype=None):
     """Explicit float64 evaluation.  Returns dict with O, LSE (log2 units, 0 at padded
-    rows) and, when ``d_out`` is given, dQ, dK, dV (all numpy float64)."""
+    rows) and, when ``d_out`` is given, dQ, dK, dV (all numpy float64).
+
+    With ``round_dtype`` (torch.float16 / torch.bfloat16) the same formulas are evaluated the way
+    a 16-bit kernel must evaluate them: the probabilities and dS are rounded to that type before
+    the second matrix products (the reference does the same: kernel.py:370, 1020, 1121, 1127), the
+    softmax denominator sums the rounded probabilities, and O is rounded before delta is formed.
+    The difference between the two evaluations is the error that rounding alone causes."""
     qn, kn, vn = (t.detach().cpu().double().numpy() for t in (q, k, v))
     B, H, T, D = qn.shape
     s = float(D) ** -0.5 if sm_scale is None else float(sm_scale)
@@ -88,6 +99,8 @@ def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=N
     row_valid = mask.any(-1, keepdims=True)                           # [B,1,T,1]
     m = np.where(row_valid, S.max(-1, keepdims=True, initial=-np.inf), 0.0)
     E = np.where(mask, np.exp(S - m), 0.0)
+    if round_dtype is not None:
+        E = _round_like(E, round_dtype)
     l = E.sum(-1, keepdims=True)
     P = np.where(row_valid, E / np.where(l == 0, 1.0, l), 0.0)
     O = np.einsum("bhij,bhjd->bhid", P, vn)
@@ -97,10 +110,18 @@ def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=N
     if d_out is not None:
         g = d_out.detach().cpu().double().numpy()
         g = np.broadcast_to(g, O.shape)
-        delta = (O * g).sum(-1, keepdims=True)
+        if round_dtype is None:
+            Pb, Ob = P, O
+        else:
+            # backward: P is rebuilt from the saved log-sum-exp and rounded for dV; O was stored rounded
+            Pb = np.where(mask, np.exp(S - lse[..., None] / LOG2E), 0.0) * row_valid
+            Ob = _round_like(O, round_dtype)
+        delta = (Ob * g).sum(-1, keepdims=True)
         dP = np.einsum("bhid,bhjd->bhij", g, vn)
-        dS = P * (dP - delta)
-        out["dV"] = np.einsum("bhij,bhid->bhjd", P, g)
+        dS = Pb * (dP - delta)
+        if round_dtype is not None:
+            Pb, dS = _round_like(Pb, round_dtype), _round_like(dS, round_dtype)
+        out["dV"] = np.einsum("bhij,bhid->bhjd", Pb, g)
         out["dQ"] = s * np.einsum("bhij,bhjd->bhid", dS, kn)
         out["dK"] = s * np.einsum("bhij,bhid->bhjd", dS, qn)
     return out

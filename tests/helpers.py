@@ -9,6 +9,13 @@ import torch
 TOL = {torch.float32: (1e-4, 0.0), torch.float16: (2e-2, 1e-2), torch.bfloat16: (2e-2, 1e-2)}
 
 
+# The log-sum-exp is a float32 output whatever the input type.  For 16-bit inputs the kernels sum the
+# ROUNDED probabilities (the weights the PV product really applies, so that they add up to one): the
+# relative error of that sum is at most the unit roundoff u of the type, i.e. at most log2(e) * u in
+# the base-2 logarithm: 7.0e-4 for float16 (u = 2^-11), 5.6e-3 for bfloat16 (u = 2^-8).
+LSE_ATOL = {torch.float32: 1e-4, torch.float16: 1e-3, torch.bfloat16: 6e-3}
+
+
 def make_inputs(B, H, T, D, seed=20, dtype=torch.float32):
     """q, k, v, dO ~ N(0,1) from a seeded CPU generator, rounded to ``dtype`` (the values the
     kernel will actually see), returned as CPU tensors of that dtype."""
@@ -39,3 +46,40 @@ def assert_close(name, got, want, dtype):
         f"{name}: {int(bad.sum())} elements out of tolerance, max abs err {err.max().item():.3e} "
         f"(atol {atol}, rtol {rtol}), worst at {np.unravel_index(int(err.argmax()), err.shape)}"
     )
+
+
+def assert_close_lse(got, want, dtype):
+    """Absolute bar of the float32 log-sum-exp output (LSE_ATOL), whatever the input type."""
+    got = torch.as_tensor(got).detach().double().cpu()
+    want = torch.as_tensor(want).detach().double().cpu()
+    assert got.shape == want.shape and torch.isfinite(got).all()
+    err = (got - want).abs().max().item() if got.numel() else 0.0
+    assert err <= LSE_ATOL[dtype], f"LSE: max abs err {err:.3e} > {LSE_ATOL[dtype]} for {dtype} inputs"
+
+
+def error_report(got, want):
+    """(max abs error, max error relative to max |want|, relative Frobenius error)."""
+    got = torch.as_tensor(got).detach().double().cpu()
+    want = torch.as_tensor(want).detach().double().cpu()
+    err = (got - want).abs()
+    scale = want.abs().max().item() or 1.0
+    fro = want.norm().item() or 1.0
+    return err.max().item(), err.max().item() / scale, (got - want).norm().item() / fro
+
+
+def assert_close_rounding_aware(name, got, exact, rounded, dtype):
+    """The BASELINE bar widened by the error that rounding P and dS to ``dtype`` causes in a
+    float64 evaluation of the same formulas: bound = atol + rtol * |exact| + 2 * max |rounded - exact|.
+    Individual rounding errors are random, so the allowance is the largest deviation anywhere in the
+    tensor, not the deviation of the same element."""
+    atol, rtol = TOL[dtype]
+    got = torch.as_tensor(got).detach().double().cpu()
+    exact = torch.as_tensor(exact).detach().double().cpu()
+    rounded = torch.as_tensor(rounded).detach().double().cpu()
+    assert torch.isfinite(got).all(), f"{name}: non-finite values"
+    allowance = 2.0 * (rounded - exact).abs().max().item()
+    err = (got - exact).abs()
+    bad = err > atol + rtol * exact.abs() + allowance
+    assert not bad.any(), (
+        f"{name}: {int(bad.sum())} elements out of tolerance, max abs err {err.max().item():.3e} "
+        f"(atol {atol}, rtol {rtol}, rounding allowance {allowance:.3e})")
