@@ -283,6 +283,55 @@ def reference_sweep(device, iters=20):
     return rows
 
 
+def tune_sweep(device, iters=10):
+    """Every variant of the 16-bit forward, dQ and dK/dV kernels (include/streaming_attention.h,
+    sa_tune_override) timed on a grid of head dimension x context_size x back_contexts, B=4, H=16,
+    T=16384 (K and V together exceed the 256 MiB last-level cache), lens = None.  The fastest variant per
+    (D, context_size class, window class) is what the library's launch-configuration table holds
+    (kernels_amd/csrc/gen_tune_table.py turns this output into the table); the reference reaches its
+    choice by autotuning at run time (src/streaming_attention/kernel.py:1154-1193)."""
+    import torch
+    from streaming_attention import _lib
+
+    lib = _lib.load()
+    B, H, T = 4, 16, 16384
+    names = {"fwd": ["narrow", "wide"], "dq": ["narrow", "wide"], "dkdv": ["blockskip", "pipelined"]}
+    rows = []
+    try:
+        for dtype_name in ("bfloat16", "float16"):
+            for D in (64, 128):
+                for C in (16, 32, 64, 128, 256, 512, 1024):
+                    for window in (512, 2048, 8192):   # one per window class of the table
+                        R = max(0, window // C - 1)
+                        if dtype_name == "float16" and window != 2048:
+                            continue   # the second type only confirms the first
+                        g = torch.Generator(device=device).manual_seed(20)
+                        dt = getattr(torch, dtype_name)
+                        q, k, v, d_o = [torch.randn(B, H, T, D, generator=g, device=device, dtype=torch.float32).to(dt)
+                                        for _ in range(4)]
+                        w = dict(q=q, k=k, v=v, d_o=d_o, lens=None, B=B, H=H, T=T, D=D, C=C, R=R, dtype=dtype_name)
+                        row = {"dtype": dtype_name, "D": D, "context_size": C, "back_contexts": R,
+                               "table": {kn: names[kn][lib.sa_launch_choice(D, C, R, ki)]
+                                         for ki, kn in enumerate(("fwd", "dq", "dkdv"))}}
+                        for ki, kn in enumerate(("fwd", "dq", "dkdv")):
+                            for vi, vn in enumerate(names[kn]):
+                                if kn == "dkdv" and vi == 1 and D != 128:
+                                    continue
+                                _lib.check(lib.sa_tune_override(ki, vi), "sa_tune_override")
+                                row[f"{kn}_{vn}_ms"] = time_kernels(w, iters)[kn]
+                            _lib.check(lib.sa_tune_override(ki, -1), "sa_tune_override")
+                        for kn in names:
+                            cand = {vn: row[f"{kn}_{vn}_ms"] for vn in names[kn] if f"{kn}_{vn}_ms" in row}
+                            row[f"{kn}_best"] = min(cand, key=cand.get)
+                        rows.append(row)
+                        del q, k, v, d_o
+    finally:
+        for ki in range(3):
+            lib.sa_tune_override(ki, -1)
+    return rows
+
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -297,6 +346,8 @@ def main():
     ap.add_argument("--zero-inputs", action="store_true",
                     help="all-zero q, k, v, dO: the same kernels and launch shapes without data-dependent "
                          "switching power (a diagnostic; the result line is marked and is not the metric)")
+    ap.add_argument("--tune-sweep", action="store_true",
+                    help="time every kernel variant on a (D, context_size, window) grid and print the rows as JSON")
     ap.add_argument("--reference-sweep", action="store_true",
                     help="time the grid of the reference's own benchmark script instead of a workload")
     args = ap.parse_args()
@@ -319,6 +370,10 @@ def main():
     if args.reference_sweep:
         print(json.dumps({"sweep": "reference benchmark grid, fp16 B=128 H=12 D=64", "n_gpus": 1,
                           "rows": reference_sweep(dev)}))
+        return
+    if args.tune_sweep:
+        print(json.dumps({"sweep": "kernel variants, B=4 H=16 T=16384, lens=None", "n_gpus": 1,
+                          "rows": tune_sweep(dev)}))
         return
     w = make_inputs(args.workload, dev, zeros=args.zero_inputs)
     B, H, T, D, C, R = w["B"], w["H"], w["T"], w["D"], w["C"], w["R"]

@@ -134,12 +134,32 @@ int sa_backward_static(const void* q, const void* k, const void* v,
  *      (1-6 describe the kernels used for float32 and for D in {16, 32, 256})
  *          7, 8: waves per workgroup of the wide / narrow forward and dQ kernels used for the
  *                16-bit types at D in {64, 128} (each wave owns 32 queries)
- *          9: smallest context_size for which the wide kernels are chosen
+ *          9: number of context_size classes of the launch-configuration table (below)
+ *         11: number of window classes of that table
  *         10: rows (B*H*T) the static workspace of sa_backward_static holds
- *         11: smallest context_size for which the software-pipelined dK/dV kernel is chosen
- *             (16-bit types, D in {64, 128})
  *   anything else: -1 */
 int sa_query(int what);
+
+/* The launch-configuration table for the 16-bit types at D in {64, 128}.  Replaces the reference's
+ * per-head-dimension tile tables and autotune spaces (src/streaming_attention/kernel.py:17-85,
+ * 1154-1193, 1212-1267): the reference searches block shapes at run time, this library ships the
+ * outcome of an offline sweep on MI355X, indexed by head dimension, context_size class
+ * (< 32, < 64, < 128, < 256, < 512, < 1024, >= 1024) and window class
+ * (context_size * (back_contexts + 1) < 1024, < 4096, >= 4096).
+ *   kernel = 0: forward   variant 0 = 4 waves (128 queries) per workgroup, 1 = 8 waves (256 queries)
+ *   kernel = 1: dQ        variant 0 = 4 waves, 1 = 8 waves
+ *   kernel = 2: dK/dV     variant 0 = block-skipping kernel, 1 = software-pipelined kernel (D = 128)
+ * sa_launch_choice() returns the variant a call with these sizes runs (-1 for a D outside {64, 128},
+ * a kernel id outside 0..2, context_size < 1 or back_contexts < 0).  Every variant computes the same
+ * function. */
+int sa_launch_choice(int D, int context_size, int back_contexts, int kernel);
+
+/* Pins one variant of one kernel for all later calls of this process, or returns to the table with
+ * variant = -1.  Meant for measurements (it is how the table was produced) and for tests that
+ * exercise every variant; the counterpart of the reference's `autotune` switch
+ * (src/streaming_attention/kernel.py:1154-1193).  A pinned dK/dV variant 1 applies to D = 128 only.
+ * Not synchronised with launches on other threads.  Returns 0 or SA_ERR_ARG. */
+int sa_tune_override(int kernel, int variant);
 
 /* Human-readable text for a return code of the functions above (static storage). */
 const char* sa_error_string(int code);

@@ -11,6 +11,10 @@ using namespace sa;
 // for the symbol; the memory is reached through the address hipGetSymbolAddress returns.
 static __device__ __align__(256) float sa_static_delta[SA_STATIC_MAX_ROWS];
 
+namespace sa {
+int g_tune_override[3] = {-1, -1, -1};
+}
+
 namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -213,11 +217,25 @@ int sa_query(int what) {
     case 6: return Cfg<__bf16>::NW * 32;
     case 7: return Cfg<__bf16>::WIDE_NW;
     case 8: return Cfg<__bf16>::NARROW_NW;
-    case 9: return Cfg<__bf16>::WIDE_CHUNK;
+    case 9: return TUNE_CHUNK_CLASSES;
     case 10: return SA_STATIC_MAX_ROWS;
-    case 11: return Cfg<__bf16>::DKDV3_MIN_CHUNK;
+    case 11: return TUNE_WINDOW_CLASSES;
   }
   return -1;
+}
+
+int sa_launch_choice(int D, int context_size, int back_contexts, int kernel) {
+  if ((D != 64 && D != 128) || context_size < 1 || back_contexts < 0 || kernel < 0 || kernel > 2) return -1;
+  const LaunchChoice c = launch_choice(D, context_size, back_contexts);
+  return kernel == 0 ? c.fwd : kernel == 1 ? c.dq : c.dkdv;
+}
+
+int sa_tune_override(int kernel, int variant) {
+  if (kernel < 0 || kernel > 2) return SA_ERR_ARG;
+  const int limit = kernel == 0 ? FWD_VARIANTS : kernel == 1 ? DQ_VARIANTS : DKDV_VARIANTS;
+  if (variant < -1 || variant >= limit) return SA_ERR_ARG;
+  g_tune_override[kernel] = variant;
+  return SA_OK;
 }
 
 const char* sa_error_string(int code) {

@@ -89,7 +89,8 @@ template <int D, int NW> static int fwd2_launch(FwdParams p, hipStream_t st) {
 template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
-    return C::wide(p.C) ? fwd2_launch<D, C::WIDE_NW>(p, st) : fwd2_launch<D, C::NARROW_NW>(p, st);
+    return launch_choice(D, p.C, p.R).fwd == FWD_WIDE ? fwd2_launch<D, C::WIDE_NW>(p, st)
+                                                      : fwd2_launch<D, C::NARROW_NW>(p, st);
   } else {
     constexpr int TQ = C::NW * 32;
     constexpr size_t lds = (size_t)2 * 2 * C::FWD_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
@@ -140,7 +141,7 @@ template <int D, int NW> static int dq2_launch(BwdParams p, hipStream_t st) {
 template <int D> static int dq_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
-    return C::wide(p.C) ? dq2_launch<D, C::WIDE_NW>(p, st) : dq2_launch<D, C::NARROW_NW>(p, st);
+    return launch_choice(D, p.C, p.R).dq == DQ_WIDE ? dq2_launch<D, C::WIDE_NW>(p, st) : dq2_launch<D, C::NARROW_NW>(p, st);
   } else {
     constexpr int TQ = C::NW * 32;
     constexpr size_t lds = (size_t)2 * 2 * C::DQ_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
@@ -187,7 +188,7 @@ template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
     // workgroup's 128 keys; that wastes nothing once a chunk holds at least those 128 keys.  Smaller
     // chunks go to the kernel whose waves skip the query tiles outside their own 32 keys' windows.
     if constexpr (D == 128) {
-      if (C::pipelined_dkdv(p.C, D)) return dkdv3_launch<D>(p, st);
+      if (launch_choice(D, p.C, p.R).dkdv == DKDV_PIPELINED) return dkdv3_launch<D>(p, st);
     }
     constexpr int TKB = C::DKDV2_NW * 32;
     constexpr size_t stages =

@@ -33,33 +33,58 @@ template <typename T, int DGROUP> int launch_dkdv(const BwdParams& p, int D, hip
 #ifndef SA_DKDV2_NST
 #define SA_DKDV2_NST 2
 #endif
-#ifndef SA_DKDV3_MIN_CHUNK
-#define SA_DKDV3_MIN_CHUNK 128
-#endif
 #ifndef SA_DKDV3_NST
 #define SA_DKDV3_NST 3
 #endif
 #ifndef SA_FWD2_NST
 #define SA_FWD2_NST 2
 #endif
+// ---- launch-configuration table -------------------------------------------------------------------
+// The 16-bit kernels for head dimensions 64 and 128 exist in several shapes; which one runs is read
+// from a table indexed by head dimension, chunk-size class and window-size class.  The entries are
+// the fastest variant measured on an MI355X at B=4, H=16, T=16384 (`bench.py --tune-sweep`, turned into
+// sa_tune_table.inc by gen_tune_table.py); float16 and bfloat16 measured alike and share the entries.
+enum FwdVariant : int { FWD_NARROW = 0,     // 4 waves (128 queries) per workgroup, two workgroups per CU
+                        FWD_WIDE = 1,       // 8 waves (256 queries) share every key tile
+                        FWD_VARIANTS = 2 };
+enum DqVariant : int { DQ_NARROW = 0, DQ_WIDE = 1, DQ_VARIANTS = 2 };
+enum DkdvVariant : int { DKDV_BLOCKSKIP = 0,   // every wave skips the query tiles outside its own 32 keys' windows
+                         DKDV_PIPELINED = 1,   // hand-scheduled loop, head dimension 128 only
+                         DKDV_VARIANTS = 2 };
+struct LaunchChoice { int fwd, dq, dkdv; };
+constexpr int TUNE_CHUNK_CLASSES = 7;    // context_size < 32, < 64, < 128, < 256, < 512, < 1024, >= 1024
+constexpr int TUNE_WINDOW_CLASSES = 3;   // context_size * (back_contexts + 1) < 1024, < 4096, >= 4096
+constexpr int chunk_class(int chunk) {
+  return chunk < 32 ? 0 : chunk < 64 ? 1 : chunk < 128 ? 2 : chunk < 256 ? 3 : chunk < 512 ? 4 : chunk < 1024 ? 5 : 6;
+}
+constexpr int window_class(int chunk, int back) {
+  const long long w = (long long)chunk * ((long long)back + 1);
+  return w < 1024 ? 0 : w < 4096 ? 1 : 2;
+}
+#include "sa_tune_table.inc"
+// Variants pinned through sa_tune_override() for measurements; -1 = use the table.
+extern int g_tune_override[3];
+inline LaunchChoice launch_choice(int D, int chunk, int back) {
+  LaunchChoice c = (D == 128 ? TUNE_D128 : TUNE_D64)[chunk_class(chunk)][window_class(chunk, back)];
+  if (g_tune_override[0] >= 0 && g_tune_override[0] < FWD_VARIANTS) c.fwd = g_tune_override[0];
+  if (g_tune_override[1] >= 0 && g_tune_override[1] < DQ_VARIANTS) c.dq = g_tune_override[1];
+  if (g_tune_override[2] >= 0 && g_tune_override[2] < DKDV_VARIANTS) c.dkdv = g_tune_override[2];
+  if (D != 128) c.dkdv = DKDV_BLOCKSKIP;
+  return c;
+}
+
 template <typename T> struct Cfg {
   static constexpr int NW = 4;                                   // waves per workgroup
   // 16-bit, D in {64, 128}: forward kernel with QB query blocks per wave and NST LDS stages
-  // The forward and dQ kernels come in two widths, chosen per call from the chunk size:
-  // 8 waves (256 queries) share each key tile among more waves, which pays once the
-  // workgroup's queries lie in one chunk; with smaller chunks the union of the waves'
-  // windows grows and 4 waves (128 queries) waste less of every tile.
+  // The forward and dQ kernels come in two widths: 8 waves (256 queries) share each key tile among
+  // more waves, which pays once the workgroup's queries lie in one chunk; with smaller chunks the
+  // union of the waves' windows grows and 4 waves (128 queries) waste less of every tile.
   static constexpr int WIDE_NW = 8, NARROW_NW = 4;
-  static constexpr int WIDE_CHUNK = 256;
-  static constexpr bool wide(int chunk) { return chunk >= WIDE_CHUNK; }
   static constexpr int DQ2_TK = SA_DQ2_TK, DQ2_NST = SA_DQ2_NST;
   static constexpr int DKDV2_NW = SA_DKDV2_NW, DKDV2_TQ = SA_DKDV2_TQ, DKDV2_NST = SA_DKDV2_NST;
-  // smallest chunk for which the software-pipelined dK/dV kernel is chosen (0x7fffffff: never)
-  static constexpr int DKDV3_MIN_CHUNK = SA_DKDV3_MIN_CHUNK;
-  // ... and only at head dimension 128: at 64 a block step has half the MFMAs for the same softmax
-  // arithmetic, the loop is bound by its vector work and dkdv2 is faster (0.23 against 0.30 ms at
-  // B=8, H=16, T=4096, chunk 128)
-  static constexpr bool pipelined_dkdv(int chunk, int D) { return D == 128 && chunk >= DKDV3_MIN_CHUNK; }
+  // The software-pipelined dK/dV kernel exists at head dimension 128 only: at 64 a block step has
+  // half the MFMAs for the same softmax arithmetic, the loop is bound by its vector work and dkdv2
+  // is faster (0.23 against 0.30 ms at B=8, H=16, T=4096, chunk 128).
   static constexpr int DKDV3_NST = SA_DKDV3_NST;
   static constexpr int FWD2_QB = SA_FWD2_QB;
   static constexpr int FWD2_NST = SA_FWD2_NST;

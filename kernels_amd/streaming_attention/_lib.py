@@ -34,6 +34,8 @@ SIGNATURES = {
                            _pi64, _pi64, _pi64, _pi64, _pi64,
                            _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp],
     "sa_query": [_i32],
+    "sa_launch_choice": [_i32, _i32, _i32, _i32],
+    "sa_tune_override": [_i32, _i32],
     "sa_error_string": [_i32],
 }
 

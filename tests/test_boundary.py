@@ -30,7 +30,7 @@ def _declared_symbols():
 def test_header_symbols_exported(lib):
     names = _declared_symbols()
     assert names == ["sa_backward", "sa_backward_static", "sa_bwd_delta", "sa_bwd_dkdv", "sa_bwd_dq", "sa_error_string",
-                     "sa_forward", "sa_query"]
+                     "sa_forward", "sa_launch_choice", "sa_query", "sa_tune_override"]
     for n in names:
         assert getattr(lib, n) is not None
     from streaming_attention import _lib
@@ -42,11 +42,25 @@ def test_query_and_error_strings(lib):
     assert lib.sa_query(0) >= 1
     assert lib.sa_query(1) in (4, 8)
     assert lib.sa_query(2) % 32 == 0 and lib.sa_query(3) % 32 == 0
-    assert (lib.sa_query(7), lib.sa_query(8)) == (8, 4) and lib.sa_query(9) == 256
+    assert (lib.sa_query(7), lib.sa_query(8)) == (8, 4) and lib.sa_query(9) == 7
     assert lib.sa_query(99) == -1
     assert b"success" in lib.sa_error_string(0)
     assert lib.sa_query(10) == 1 << 21
-    assert lib.sa_query(11) == 128
+    assert lib.sa_query(11) == 3 and lib.sa_query(12) == -1
+    # the launch-configuration table answers without a GPU and rejects what it does not cover
+    for D in (64, 128):
+        for C in (1, 31, 32, 100, 256, 5000):
+            for R in (0, 3, 100, 2 ** 31 - 1):
+                assert lib.sa_launch_choice(D, C, R, 0) in (0, 1)
+                assert lib.sa_launch_choice(D, C, R, 1) in (0, 1)
+                assert lib.sa_launch_choice(D, C, R, 2) in ((0, 1) if D == 128 else (0,))
+    assert lib.sa_launch_choice(32, 64, 1, 0) == -1 and lib.sa_launch_choice(128, 0, 1, 0) == -1
+    assert lib.sa_launch_choice(128, 64, 1, 3) == -1 and lib.sa_launch_choice(128, 64, -1, 0) == -1
+    assert lib.sa_tune_override(0, 2) == -3 and lib.sa_tune_override(3, 0) == -3
+    assert lib.sa_tune_override(0, 1) == 0 and lib.sa_launch_choice(64, 8, 0, 0) == 1
+    assert lib.sa_tune_override(2, 1) == 0 and lib.sa_launch_choice(64, 512, 0, 2) == 0
+    for k in range(3):
+        assert lib.sa_tune_override(k, -1) == 0
     for code in (-1, -2, -3, -4, -5, -6):
         assert len(lib.sa_error_string(code)) > 10
 

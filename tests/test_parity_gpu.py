@@ -130,6 +130,43 @@ def test_tile_edges_16bit(T, C, R, dtype):
     check_against_dense(q, k, v, d_o, lens, C, R, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("C,R", [(16, 2), (48, 30), (100, 3), (200, 1), (300, 4), (600, 0), (1100, 1)])
+def test_every_table_class_16bit(C, R, D, dtype):
+    """One context_size per class of the launch-configuration table, windows in all three window
+    classes, run with the variants the table picks."""
+    B, H, T = 2, 2, 1500
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=31, dtype=dtype)
+    lens = torch.tensor([T, T - 333], dtype=torch.int32)
+    check_against_dense(q, k, v, d_o, lens, C, R, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("D", [64, 128])
+def test_every_kernel_variant_16bit(D, dtype):
+    """Each variant of the forward, dQ and dK/dV kernels pinned in turn (sa_tune_override), on chunk
+    sizes below, at and above the workgroups' 128 / 256 rows; all must agree with the oracle."""
+    from streaming_attention import _lib
+
+    lib = _lib.load()
+    B, H, T = 2, 2, 777
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=32, dtype=dtype)
+    lens = torch.tensor([T, 500], dtype=torch.int32)
+    n_variants = (2, 2, 2 if D == 128 else 1)
+    try:
+        for kernel in range(3):
+            for variant in range(n_variants[kernel]):
+                assert lib.sa_tune_override(kernel, variant) == 0
+                for C, R in ((24, 5), (128, 2), (256, 1), (320, 8)):
+                    assert lib.sa_launch_choice(D, C, R, kernel) == variant
+                    check_against_dense(q, k, v, d_o, lens, C, R, dtype)
+            assert lib.sa_tune_override(kernel, -1) == 0
+    finally:
+        for kernel in range(3):
+            lib.sa_tune_override(kernel, -1)
+
+
 def test_golden_vectors():
     data = np.load(GOLDEN, allow_pickle=False)
     for name in sorted({k.split(".")[0] for k in data.files}):
