@@ -332,6 +332,40 @@ def tune_sweep(device, iters=10):
 
 
 
+def path_sweep(device, iters=10):
+    """Per-kernel times of every (dtype, head dimension) family the library serves, on one shape
+    (B=4, H=16, T=4096, context_size=128, back_contexts=4, lens=None): the 16-bit D in {64, 128}
+    kernels next to the first-generation kernels that serve float32 and D in {16, 32, 256}
+    (the reference covers the same range from one tuned kernel, src/streaming_attention/kernel.py:196-203,
+    1288-1290).  Rates are executed flop (S and dP are computed by both backward kernels) and
+    algorithmic HBM bytes."""
+    import torch
+
+    B, H, T, C, R = 4, 16, 4096, 128, 4
+    P = unmasked_pairs(T, C, R, [T] * B)
+    rows = []
+    for dtype_name in ("float32", "float16", "bfloat16"):
+        for D in (16, 32, 64, 128, 256):
+            dt = getattr(torch, dtype_name)
+            g = torch.Generator(device=device).manual_seed(20)
+            q, k, v, d_o = [(torch.randn(B, H, T, D, generator=g, device=device, dtype=torch.float32) * D ** -0.25).to(dt)
+                            for _ in range(4)]
+            w = dict(q=q, k=k, v=v, d_o=d_o, lens=None, B=B, H=H, T=T, D=D, C=C, R=R, dtype=dtype_name)
+            kt = time_kernels(w, iters)
+            es = 4 if dtype_name == "float32" else 2
+            tensor, stat = float(B * H * T) * D * es, 4.0 * B * H * T
+            fl = {"fwd": 4.0 * D * H * P, "dq": 6.0 * D * H * P, "dkdv": 8.0 * D * H * P}
+            by = {"fwd": 4 * tensor + stat, "delta": 2 * tensor + stat, "dq": 5 * tensor + 2 * stat,
+                  "dkdv": 6 * tensor + 2 * stat}
+            rows.append({"dtype": dtype_name, "D": D, "kernel_ms": kt,
+                         "kernel_tflops": {n: fl[n] / (kt[n] * 1e-3) / 1e12 for n in fl},
+                         "kernel_gbs": {n: by[n] / (kt[n] * 1e-3) / 1e9 for n in by},
+                         "fwd_bwd_effective_tflops": 14.0 * D * H * P / (sum(kt.values()) * 1e-3) / 1e12})
+            del q, k, v, d_o
+    return rows
+
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -346,6 +380,8 @@ def main():
     ap.add_argument("--zero-inputs", action="store_true",
                     help="all-zero q, k, v, dO: the same kernels and launch shapes without data-dependent "
                          "switching power (a diagnostic; the result line is marked and is not the metric)")
+    ap.add_argument("--path-sweep", action="store_true",
+                    help="time the kernels of every (dtype, head dimension) family on one shape and print the rows as JSON")
     ap.add_argument("--tune-sweep", action="store_true",
                     help="time every kernel variant on a (D, context_size, window) grid and print the rows as JSON")
     ap.add_argument("--reference-sweep", action="store_true",
@@ -370,6 +406,10 @@ def main():
     if args.reference_sweep:
         print(json.dumps({"sweep": "reference benchmark grid, fp16 B=128 H=12 D=64", "n_gpus": 1,
                           "rows": reference_sweep(dev)}))
+        return
+    if args.path_sweep:
+        print(json.dumps({"sweep": "dtype x head dimension, B=4 H=16 T=4096 context_size=128 back_contexts=4", "n_gpus": 1,
+                          "rows": path_sweep(dev)}))
         return
     if args.tune_sweep:
         print(json.dumps({"sweep": "kernel variants, B=4 H=16 T=16384, lens=None", "n_gpus": 1,
