@@ -21,17 +21,20 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// strides are element counts; dim stride 1, the others whole 16-byte vectors
-// and the kernels address rows of one (batch, head) slice with 32-bit byte offsets
-int check_layout(const void* p, const int64_t* s, int dtype, int T) {
+// strides are element counts; dim stride 1, the others whole 16-byte vectors.  The 16-bit kernels
+// for D in {64, 128} address the rows of one (batch, head) slice with 32-bit byte offsets through a
+// buffer descriptor; the others compute 64-bit addresses and have no such limit.  A zero stride along
+// T (one row repeated) is refused: no caller needs it and no test covers it.
+int check_layout(const void* p, const int64_t* s, int dtype, int T, int D) {
   if (!p || !s) return SA_ERR_ARG;
   const int64_t vec = dtype == SA_DTYPE_F32 ? 4 : 8;
   if (s[3] != 1) return SA_ERR_LAYOUT;
   if (!aligned16(p)) return SA_ERR_LAYOUT;
   for (int i = 0; i < 3; ++i)
     if (s[i] % vec != 0) return SA_ERR_LAYOUT;
-  if (s[2] < 0) return SA_ERR_LAYOUT;
-  if (((int64_t)T + 1024) * s[2] * (dtype == SA_DTYPE_F32 ? 4 : 2) >= (int64_t(1) << 32)) return SA_ERR_TOO_LARGE;
+  if (s[2] < 0 || (s[2] == 0 && T > 1)) return SA_ERR_LAYOUT;
+  const bool offsets32 = dtype != SA_DTYPE_F32 && (D == 64 || D == 128);
+  if (offsets32 && ((int64_t)T + 1024) * s[2] * 2 >= (int64_t(1) << 32)) return SA_ERR_TOO_LARGE;
   return SA_OK;
 }
 
@@ -67,9 +70,9 @@ int sa_forward(const void* q, const void* k, const void* v, const int32_t* lens,
   if (int rc = check_common(B, H, T, D, dtype)) return rc;
   if (context_size < 1 || back_contexts < 0) return SA_ERR_ARG;
   if (B == 0 || H == 0 || T == 0) return SA_OK;
-  if (int rc = check_layout(q, qs, dtype, T)) return rc;
-  if (int rc = check_layout(k, ks, dtype, T)) return rc;
-  if (int rc = check_layout(v, vs, dtype, T)) return rc;
+  if (int rc = check_layout(q, qs, dtype, T, D)) return rc;
+  if (int rc = check_layout(k, ks, dtype, T, D)) return rc;
+  if (int rc = check_layout(v, vs, dtype, T, D)) return rc;
   if (!o || !aligned16(o)) return o ? SA_ERR_LAYOUT : SA_ERR_ARG;
   FwdParams p{};
   p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse; p.lens = lens; p.lens_stride = lens_stride;
@@ -88,8 +91,8 @@ int sa_bwd_delta(const void* o, const void* d_o, float* delta, const int64_t* os
                  int H, int T, int D, int dtype, void* stream) {
   if (int rc = check_common(B, H, T, D, dtype)) return rc;
   if (B == 0 || H == 0 || T == 0) return SA_OK;
-  if (int rc = check_layout(o, os, dtype, T)) return rc;
-  if (int rc = check_layout(d_o, gs, dtype, T)) return rc;
+  if (int rc = check_layout(o, os, dtype, T, D)) return rc;
+  if (int rc = check_layout(d_o, gs, dtype, T, D)) return rc;
   if (!delta) return SA_ERR_ARG;
   DeltaParams p{};
   p.o = o; p.d_o = d_o; p.delta = delta;
@@ -108,10 +111,10 @@ static int fill_bwd(BwdParams& p, const void* q, const void* k, const void* v, c
   if (int rc = check_common(B, H, T, D, dtype)) return rc;
   if (context_size < 1 || back_contexts < 0) return SA_ERR_ARG;
   if (B == 0 || H == 0 || T == 0) return SA_OK;
-  if (int rc = check_layout(q, qs, dtype, T)) return rc;
-  if (int rc = check_layout(k, ks, dtype, T)) return rc;
-  if (int rc = check_layout(v, vs, dtype, T)) return rc;
-  if (int rc = check_layout(d_o, gs, dtype, T)) return rc;
+  if (int rc = check_layout(q, qs, dtype, T, D)) return rc;
+  if (int rc = check_layout(k, ks, dtype, T, D)) return rc;
+  if (int rc = check_layout(v, vs, dtype, T, D)) return rc;
+  if (int rc = check_layout(d_o, gs, dtype, T, D)) return rc;
   if (!lse || !delta) return SA_ERR_ARG;
   p.q = q; p.k = k; p.v = v; p.d_o = d_o; p.lse = lse; p.delta = delta;
   p.lens = lens; p.lens_stride = lens_stride;

@@ -4,8 +4,8 @@ Same dispatcher names, argument lists, fake implementations and autograd registr
 the reference (src/streaming_attention/kernel.py:1270-1530); the bodies enqueue the HIP
 kernels of libstreaming_attention.so on the current stream instead of launching Triton
 kernels.  ``autotune``, ``prescale_qk`` and ``precision`` are accepted for signature
-compatibility and do not change the result: tile shapes are fixed per (dtype, head_dim)
-and all accumulation is fp32.
+compatibility and do not change the result: kernel variants are read from a table measured
+on MI355X (head dimension, context_size class, window class) and all accumulation is fp32.
 """
 from __future__ import annotations
 
@@ -28,19 +28,22 @@ def _dtype_id(dtype: torch.dtype) -> int:
 
 def _kernel_layout(t: torch.Tensor) -> torch.Tensor:
     """Return ``t`` itself when the kernels can read it in place (unit stride along the head
-    dimension, every other stride and the base address a multiple of 16 bytes), otherwise a
-    contiguous copy.  The kernels address the rows of one (batch, head) slice with 32-bit
-    byte offsets (a contiguous tensor is within that range up to tens of millions of positions)."""
+    dimension, every other stride and the base address a multiple of 16 bytes, a non-zero stride
+    along T), otherwise a contiguous copy.  The 16-bit kernels for head dimensions 64 and 128
+    address the rows of one (batch, head) slice with 32-bit byte offsets (a contiguous tensor is
+    within that range up to tens of millions of positions); the other kernels have no such limit."""
     es = t.element_size()
+    offsets32 = es == 2 and t.shape[-1] in (64, 128)
     if t.is_contiguous() and t.data_ptr() % _VEC_BYTES == 0 and t.shape[-1] * es % _VEC_BYTES == 0 \
-            and (t.shape[-2] + 1024) * t.shape[-1] * es < 2**32:
+            and (not offsets32 or (t.shape[-2] + 1024) * t.shape[-1] * es < 2**32):
         return t          # the common case, without looking at every stride
     vec = _VEC_BYTES // es
     ok = (
         t.stride(-1) == 1
         and all(s % vec == 0 for s in t.stride()[:-1])
+        and (t.stride(-2) > 0 or t.shape[-2] <= 1)
         and t.data_ptr() % _VEC_BYTES == 0
-        and (t.shape[-2] + 1024) * t.stride(-2) * es < 2**32
+        and (not offsets32 or (t.shape[-2] + 1024) * t.stride(-2) * es < 2**32)
     )
     return t if ok else t.contiguous()
 

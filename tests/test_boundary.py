@@ -87,6 +87,7 @@ def test_validation_codes_without_gpu(lib):
     assert fwd(qs=(ctypes.c_int64 * 4)(8192, 1024, 64, 2)) == -4   # dim stride != 1
     assert fwd(qs=(ctypes.c_int64 * 4)(8192, 1024, 63, 1)) == -4   # row stride not a whole vector
     assert fwd(T=2**22, qs=(ctypes.c_int64 * 4)(2**33, 64, 2048, 1)) == -5   # row offsets beyond 32 bits
+    assert fwd(qs=(ctypes.c_int64 * 4)(8192, 1024, 0, 1)) == -4    # one row repeated along T
     assert fwd(B=0) == 0 and fwd(T=0) == 0                         # empty problems are no-ops
     assert lib.sa_bwd_delta(p, p, None, st, st, 1, 1, 8, 64, 2, None) == -3
     # the static-workspace backward refuses what its array cannot hold, before any HIP call

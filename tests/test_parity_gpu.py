@@ -167,6 +167,34 @@ def test_every_kernel_variant_16bit(D, dtype):
             lib.sa_tune_override(kernel, -1)
 
 
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 64), (torch.float16, 64), (torch.bfloat16, 128), (torch.float16, 32)],
+                         ids=str)
+def test_expanded_heads_and_repeated_rows(dtype, D):
+    """k and v expanded over the head axis (stride 0, read in place: multi-query attention without a
+    copy) and a v that repeats one row along T (stride 0 along T: the host makes a contiguous copy)."""
+    from streaming_attention import streaming_attention
+
+    dev = torch.device("cuda:0")
+    B, H, T, C, R = 2, 4, 200, 32, 2
+    q, k1, v1, d_o = make_inputs(B, H, T, D, seed=33, dtype=dtype)
+    k1, v1 = k1[:, :1], v1[:, :1]
+    lens = torch.tensor([T, 77], dtype=torch.int32)
+    for v_src in (v1, v1[:, :, :1].expand(B, 1, T, D)):
+        qd = q.to(dev).requires_grad_()
+        kd, vd = k1.to(dev).requires_grad_(), v_src.to(dev).requires_grad_()
+        ke, ve = kd.expand(B, H, T, D), vd.expand(B, H, T, D)
+        assert ke.stride(1) == 0
+        o = streaming_attention(qd, ke, ve, lens.to(dev), C, R)
+        o.backward(d_o.to(dev))
+        ref = sa_oracle.dense_f64(q, k1.expand(B, H, T, D), v_src.expand(B, H, T, D), lens, C, R, d_out=d_o)
+        assert_close("O", o.detach(), ref["O"], dtype)
+        assert_close("dQ", qd.grad, ref["dQ"], dtype)
+        # autograd sums the per-head gradients of the expanded tensors (in the element type, so the
+        # bar widens with the number of heads summed)
+        assert_close("dK", kd.grad.double().cpu() / H, ref["dK"].sum(1, keepdims=True) / H, dtype)
+        assert_close("dV", vd.grad.double().cpu() / H, ref["dV"].sum(1, keepdims=True) / H, dtype)
+
+
 def test_golden_vectors():
     data = np.load(GOLDEN, allow_pickle=False)
     for name in sorted({k.split(".")[0] for k in data.files}):
