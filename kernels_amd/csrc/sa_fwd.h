@@ -216,9 +216,6 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
 // rate); K and V tiles are brought in by asynchronous global->LDS copies into a ring of NST
 // stages, NST-1 tiles ahead of the compute, with one barrier per key tile.
 template <typename T, int D, int QB, int NW, int TK, int NST>
-#ifdef SA_FWD2_WPE
-__attribute__((amdgpu_waves_per_eu(SA_FWD2_WPE)))
-#endif
 __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   using E = Elem<T>;
   using G = TileGeom<T, D>;
