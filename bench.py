@@ -295,7 +295,7 @@ def tune_sweep(device, iters=10):
 
     lib = _lib.load()
     B, H, T = 4, 16, 16384
-    names = {"fwd": ["narrow", "wide"], "dq": ["narrow", "wide"], "dkdv": ["blockskip", "pipelined"]}
+    names = {"fwd": ["narrow", "wide"], "dq": ["narrow", "wide", "pipelined"], "dkdv": ["blockskip", "pipelined"]}
     rows = []
     try:
         for dtype_name in ("bfloat16", "float16"):
@@ -315,7 +315,7 @@ def tune_sweep(device, iters=10):
                                          for ki, kn in enumerate(("fwd", "dq", "dkdv"))}}
                         for ki, kn in enumerate(("fwd", "dq", "dkdv")):
                             for vi, vn in enumerate(names[kn]):
-                                if kn == "dkdv" and vi == 1 and D != 128:
+                                if vn == "pipelined" and D != 128:
                                     continue
                                 _lib.check(lib.sa_tune_override(ki, vi), "sa_tune_override")
                                 row[f"{kn}_{vn}_ms"] = time_kernels(w, iters)[kn]

@@ -147,7 +147,7 @@ int sa_query(int what);
  * (< 32, < 64, < 128, < 256, < 512, < 1024, >= 1024) and window class
  * (context_size * (back_contexts + 1) < 1024, < 4096, >= 4096).
  *   kernel = 0: forward   variant 0 = 4 waves (128 queries) per workgroup, 1 = 8 waves (256 queries)
- *   kernel = 1: dQ        variant 0 = 4 waves, 1 = 8 waves
+ *   kernel = 1: dQ        variant 0 = 4 waves, 1 = 8 waves, 2 = software-pipelined kernel (D = 128)
  *   kernel = 2: dK/dV     variant 0 = block-skipping kernel, 1 = software-pipelined kernel (D = 128)
  * sa_launch_choice() returns the variant a call with these sizes runs (-1 for a D outside {64, 128},
  * a kernel id outside 0..2, context_size < 1 or back_contexts < 0).  Every variant computes the same
@@ -157,7 +157,7 @@ int sa_launch_choice(int D, int context_size, int back_contexts, int kernel);
 /* Pins one variant of one kernel for all later calls of this process, or returns to the table with
  * variant = -1.  Meant for measurements (it is how the table was produced) and for tests that
  * exercise every variant; the counterpart of the reference's `autotune` switch
- * (src/streaming_attention/kernel.py:1154-1193).  A pinned dK/dV variant 1 applies to D = 128 only.
+ * (src/streaming_attention/kernel.py:1154-1193).  A pinned software-pipelined variant applies to D = 128 only.
  * Not synchronised with launches on other threads.  Returns 0 or SA_ERR_ARG. */
 int sa_tune_override(int kernel, int variant);
 

@@ -9,6 +9,7 @@
 #else
 #include "sa_bwd.h"
 #include "sa_bwd3.h"
+#include "sa_bwd4.h"
 #endif
 
 namespace sa {
@@ -138,9 +139,32 @@ template <int D, int NW> static int dq2_launch(BwdParams p, hipStream_t st) {
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), lds, st, p);
   return (int)hipGetLastError();
 }
+// hand-scheduled loop, one wave per SIMD, 64 queries per wave (head dimension 128)
+template <int D> static int dq3_launch(BwdParams p, hipStream_t st) {
+  using C = Cfg<ElemT>;
+  if constexpr (C::fwd2(D) && D == 128) {
+    constexpr int NW = 4, TQ = NW * 64, NST = 4;
+    constexpr size_t stages = (size_t)NST * 2 * 64 * D * sizeof(ElemT);
+    constexpr size_t patches = (size_t)NW * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
+    constexpr size_t lds = stages > patches ? stages : patches;
+    auto kern = dq3_kernel<ElemT, D, NST>;
+    static PrepareState once;
+    if (int rc = prepare(kern, lds, once)) return rc;
+    p.n_tiles = (int)ceil_div(p.T, TQ);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+  } else {
+    return SA_ERR_HEAD_DIM;
+  }
+}
 template <int D> static int dq_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
+    if constexpr (D == 128) {
+      if (launch_choice(D, p.C, p.R).dq == DQ_PIPELINED) return dq3_launch<D>(p, st);
+    }
     return launch_choice(D, p.C, p.R).dq == DQ_WIDE ? dq2_launch<D, C::WIDE_NW>(p, st) : dq2_launch<D, C::NARROW_NW>(p, st);
   } else {
     constexpr int TQ = C::NW * 32;

@@ -47,7 +47,9 @@ template <typename T, int DGROUP> int launch_dkdv(const BwdParams& p, int D, hip
 enum FwdVariant : int { FWD_NARROW = 0,     // 4 waves (128 queries) per workgroup, two workgroups per CU
                         FWD_WIDE = 1,       // 8 waves (256 queries) share every key tile
                         FWD_VARIANTS = 2 };
-enum DqVariant : int { DQ_NARROW = 0, DQ_WIDE = 1, DQ_VARIANTS = 2 };
+enum DqVariant : int { DQ_NARROW = 0, DQ_WIDE = 1,
+                       DQ_PIPELINED = 2,   // hand-scheduled loop, 4 waves of 64 queries (head dimension 128 only)
+                       DQ_VARIANTS = 3 };
 enum DkdvVariant : int { DKDV_BLOCKSKIP = 0,   // every wave skips the query tiles outside its own 32 keys' windows
                          DKDV_PIPELINED = 1,   // hand-scheduled loop, head dimension 128 only
                          DKDV_VARIANTS = 2 };
@@ -70,6 +72,7 @@ inline LaunchChoice launch_choice(int D, int chunk, int back) {
   if (g_tune_override[1] >= 0 && g_tune_override[1] < DQ_VARIANTS) c.dq = g_tune_override[1];
   if (g_tune_override[2] >= 0 && g_tune_override[2] < DKDV_VARIANTS) c.dkdv = g_tune_override[2];
   if (D != 128) c.dkdv = DKDV_BLOCKSKIP;
+  if (D != 128 && c.dq == DQ_PIPELINED) c.dq = DQ_NARROW;
   return c;
 }
 
