@@ -36,12 +36,8 @@ Register map (D = 128):
 Run:  python3 gen_dq3_asm.py > sa_dq3_asm.inc   (the Makefile does this)
 """
 
-import os
-
-ABLATE = os.environ.get("DQ3_ABLATE", "")   # timing experiments only: v = no vector arithmetic, l = no LDS reads, m = no MFMAs
-
 RING = 8
-PF = 3 if "p" in ABLATE else RING - 1          # fragments between a read and its use
+PF = RING - 1          # fragments between a read and its use
 NFRAG = 24             # fragments per iteration: 8 K rows, 8 V rows (alternating), 8 K transposed
 NSLOT = 48
 ROWB = 256
@@ -102,13 +98,9 @@ class Gen:
         self.tails = []      # out-of-line blocks
 
     def emit(self, s):
-        if "m" in ABLATE and s.startswith("v_mfma"):
-            return
         self.out.append(s)
 
     def lds(self, tag, text):
-        if "l" in ABLATE or ("r" in ABLATE and "ds_read_b128" in text) or ("t" in ABLATE and "_tr_" in text):
-            return
         self.issued.append(tag)
         self.emit(text)
 
@@ -207,10 +199,6 @@ class Gen:
         iterations: the tile hand-over)."""
         self.out = []
         vops = self.vector_ops(par, lab)
-        if "v" in ABLATE:
-            vops = [f"Lmaskback_{lab}:"]
-        if "e" in ABLATE:
-            vops = [op for op in vops if isinstance(op, tuple) or not op.startswith("v_exp")]
         if par == 0:
             # row addresses move to the next tile after this iteration's own last row read (slot 16
             # issues it) and after the hand-over, before slot 34 reads the next iteration's first
@@ -316,11 +304,11 @@ def generate(dt):
         return ["s_add_i32 s66, s42, 1",
                 "s_cmp_ge_i32 s66, s41",
                 f"s_cbranch_scc1 Lskip_{lab}",
-                "s_waitcnt vmcnt(0)" if "b" not in ABLATE else "s_nop 0",
-                "s_barrier" if "b" not in ABLATE else "s_nop 0",
+                "s_waitcnt vmcnt(0)",
+                "s_barrier",
                 "s_add_i32 s66, s42, 2",
                 "s_cmp_ge_i32 s66, s41",
-                f"s_cbranch_scc1 Lskip_{lab}"] + (issue_tile() if "d" not in ABLATE else []) + [f"Lskip_{lab}:"]
+                f"s_cbranch_scc1 Lskip_{lab}"] + issue_tile() + [f"Lskip_{lab}:"]
     k = 1
     first = g.body(k, 0, L("f"), with_dq=False, mid=mid(L("f")))
     k += 1
