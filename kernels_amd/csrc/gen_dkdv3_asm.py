@@ -11,8 +11,8 @@ and the hazards the hardware leaves to software spaced out by construction.
 Register map (the kernel is built for D = 128):
   a[0:63]    dV^T blocks (16 registers per 32 columns of D)     a[64:127]  dK^T blocks
   a[128:159] K fragments (4 registers per 16 columns of D)      a[160:191] V fragments (negated)
-  v[0:31]    score accumulators of the even / odd block         v[32:63]   delta - dP accumulators
-  v[64:79]   probabilities, then -dS, of the current block      v[80:95]   lse of the next block's rows
+  v[0:31]    lse - score accumulators of the even / odd block   v[32:63]   delta - dP accumulators
+  v[64:79]   probabilities, then -dS, of the current block      v[80:95]   free
   v[96:103]  P rounded (two B operands)                         v[104:111] -dS rounded
   v[112:143] fragment ring, 8 entries of 4 registers
   v[144:151] row-fragment addresses, tile of the B side         v[152:159] same, next tile
@@ -23,7 +23,7 @@ Register map (the kernel is built for D = 128):
   v[208:239] wave-uniform inputs, copied to s40... at entry (see SCALARS below)
   v240, v241 buffer offsets of this lane for the Q / dO tile loads    v[242:243] lse (lanes 0-15) or delta
   (lanes 16-31) row pointer    v244 row of the next tile this lane fetches lse / delta for    v[245:247] temporaries
-  s40 |scale*log2e|  s41 one past the last query tile  s42 query tile of the B side  s43 64*s42  s44 first row of
+  s40 free  s41 one past the last query tile  s42 query tile of the B side  s43 64*s42  s44 first row of
   the block being masked  s45..s47 LDS address of the stages of tiles s42, s42+1, s42+2  s48 wave offset inside a
   tile for the asynchronous loads  s49 same for lse/delta  s50 last valid row  s[52:55], s[56:59] buffer resources
   of Q and dO  s60, s61 their running byte offsets  s62, s63 bytes between a wave's load instructions
@@ -71,9 +71,6 @@ class Gen:
 
     def PR(self, i):
         return self.vr(64 + i)
-
-    def LR(self, i):
-        return self.vr(80 + i)
 
     def PB(self, half, w=None):
         return self.vr(96 + 4 * half, 4) if w is None else self.vr(96 + 4 * half + w)
@@ -146,25 +143,20 @@ class Gen:
         return ((r // RPW) * 2 * RPW + (r % RPW) + which * RPW) * 4
 
     # ---- vector work ---------------------------------------------------------------------------
-    def v1_ops(self, par, blk):
-        """Probabilities of block `blk` (scores in S[par]): per element fma -> exp, rounding per pair.
-        Returns one list of instructions per element step; a v_exp result is never consumed by the
-        very next instruction (transcendental forwarding needs one instruction in between)."""
-        def fma(i):
-            return [("need", ("lse", blk, i >> 2)),
-                    f"v_fma_f32 {self.PR(i)}, {self.S(par, i)}, s40, -{self.LR(i)}"]
+    def v1_ops(self, par):
+        """Probabilities of the block whose accumulator S[par] holds lse - score*scale*log2(e):
+        P = exp2(-S), rounded per pair.  Returns one list of instructions per element step; a v_exp
+        result is never consumed by the very next instruction (transcendental forwarding needs one
+        instruction in between), so a pair is rounded after the exponential of the next element."""
+        def cvt(i):     # pair (i - 1, i)
+            return f"{self.cvt} {self.PB(i >> 3, (i & 7) >> 1)}, {self.PR(i - 1)}, {self.PR(i)}"
         steps = []
         for i in range(16):
-            ops = []
-            if i == 0:
-                ops += fma(0) + fma(1)
-            ops.append(f"v_exp_f32 {self.PR(i)}, {self.PR(i)}")
-            if i + 2 < 16:
-                ops += fma(i + 2)
-            if i & 1:
-                if i + 2 >= 16:
-                    ops.append("s_nop 0")
-                ops.append(f"{self.cvt} {self.PB(i >> 3, (i & 7) >> 1)}, {self.PR(i - 1)}, {self.PR(i)}")
+            ops = [f"v_exp_f32 {self.PR(i)}, -{self.S(par, i)}"]
+            if i >= 2 and (i & 1) == 0:
+                ops.append(cvt(i - 1))
+            if i == 15:
+                ops += ["s_nop 0", cvt(15)]
             steps.append(ops)
         return steps
 
@@ -177,10 +169,11 @@ class Gen:
         return steps
 
     def mask_ops(self, par):
-        """S[par] = 0 where (row, this lane's key) is inside the key's window, -inf elsewhere,
-        for the block whose first row is s44."""
+        """S[par] keeps its value (the lse of the row) where (row, this lane's key) is inside the
+        key's window and becomes +inf elsewhere, for the block whose first row is s44."""
         t = self.TMP
-        ops = [f"v_subrev_u32 v{t}, s44, v{self.QLO}",
+        ops = ["s_mov_b32 s67, 0x7f800000",
+               f"v_subrev_u32 v{t}, s44, v{self.QLO}",
                f"v_subrev_u32 v{t + 1}, s44, v{self.QHI}",
                f"v_med3_i32 v{t}, v{t}, 0, 32",
                f"v_med3_i32 v{t + 1}, v{t + 1}, 0, 32",
@@ -190,18 +183,18 @@ class Gen:
                f"v_add_u32 v{t + 4}, -1, v{t + 4}",
                f"v_not_b32 v{t + 2}, v{t + 2}",
                f"v_and_b32 v{t + 4}, v{t + 4}, v{t + 2}",
-               f"v_lshrrev_b32 v{t + 4}, v{self.H4}, v{t + 4}",
-               f"v_not_b32 v{t + 6}, v{t + 4}"]
-        # bit -> all-ones / zero with v_bfe_i32 into one of four temporaries; the v_and that uses it
+               f"v_lshrrev_b32 v{t + 4}, v{self.H4}, v{t + 4}"]
+        # bit -> all-ones / zero with v_bfe_i32 into one of four temporaries; the select that uses it
         # is issued three elements later, before that temporary is written again
+        def sel(k):
+            return f"v_bitop3_b32 {self.S(par, k)}, {self.S(par, k)}, s67, v{t + 7 + (k & 3)} bitop3:0xe4"
         for i in range(16):
             pos = 8 * (i >> 2) + (i & 3)
-            ops.append(f"v_bfe_i32 v{t + 7 + (i & 3)}, v{t + 6}, {pos}, 1")
+            ops.append(f"v_bfe_i32 v{t + 7 + (i & 3)}, v{t + 4}, {pos}, 1")
             if i >= 3:
-                k = i - 3
-                ops.append(f"v_and_b32 {self.S(par, k)}, 0xff800000, v{t + 7 + (k & 3)}")
+                ops.append(sel(i - 3))
         for k in range(13, 16):
-            ops.append(f"v_and_b32 {self.S(par, k)}, 0xff800000, v{t + 7 + (k & 3)}")
+            ops.append(sel(k))
         return ops
 
     # ---- one block step ---------------------------------------------------------------------
@@ -210,7 +203,7 @@ class Gen:
         instruction lists per part (two parts when split_at is given)."""
         NA, NB, NS, DB = self.NA, self.NB, self.NS, self.DB
         parts, self.out = [], []
-        v1 = self.v1_ops(par, k)
+        v1 = self.v1_ops(par)
         v2 = self.v2_ops(par)
         mask = self.mask_ops(par)
         # address work of an odd step: this tile <- next tile, next tile and B side recomputed
@@ -221,8 +214,6 @@ class Gen:
         tail = [f"v_mov_b32 v{self.ALD_CUR}, v{self.ALD_NXT}",
                 f"v_add_u32 v{self.ALD_NXT}, s47, v{self.ALD_BASE}"]
         eps, epv = 16 // NA, 16 // NB
-        zero = [f"v_mov_b32 {self.S(par, i)}, 0" for i in range(16)]
-        nz = -(-16 // NB)
         for j in range(NS):
             if split_at is not None and j == split_at:
                 parts.append(self.out)
@@ -243,13 +234,12 @@ class Gen:
                         self.need(("delta", k + 1, 3))
                     self.emit(f"{self.mfma} {self.DP(par ^ 1)}, {self.RG(r)}, {self.VF(g)}, {self.DP(par ^ 1)}")
                 else:
+                    if j == 0:
+                        self.need(("lse", k + 1, 3))
                     self.emit(f"{self.mfma} {self.S(par ^ 1)}, {self.RG(r)}, {self.KF(g)}, {self.S(par ^ 1)}")
                 for e in range(j * eps, (j + 1) * eps):
                     for op in v1[e]:
-                        if isinstance(op, tuple):
-                            self.need(op[1])
-                        else:
-                            self.emit(op)
+                        self.emit(op)
             elif j < NA + NB:
                 idx = j - NA
                 half, m = idx // DB, idx % DB
@@ -263,33 +253,23 @@ class Gen:
                 idx = j - NA - NB
                 half, m = idx // DB, idx % DB
                 self.emit(f"{self.mfma} {self.DK(m)}, {self.RG(r)}, {self.DSB(half)}, {self.DK(m)}")
-                # row statistics: delta of block k + 2 starts its dP accumulator, lse of block k + 1
-                # feeds the next A phase.  They read the next tile, so they come after the point
-                # where an even step waits for it.
+                # row statistics of block k + 2, which has this step's parity (block `par` of the next
+                # tile; for an odd step: of the tile that becomes "this tile" when it rotates its
+                # addresses): its lse starts the score accumulator, its delta the dP accumulator.
+                # They read the next tile, so they come after the point where an even step waits for
+                # it, two per slot, lse first: the next step's first MFMA reads it.
                 i0 = max(0, (NS - PF) - (NA + NB))
-                slots_r = NB - i0
-                base_n, extra = 8 // slots_r, 8 % slots_r
-                if idx >= i0:
-                    q = idx - i0
-                    first = q * base_n + min(q, extra)
-                    count = base_n + (1 if q < extra else 0)
-                else:
-                    first, count = 0, 0
-                for rr in range(first, first + count):
-                    if rr < 4:
-                        # block k + 2 has this step's parity: block `par` of the next tile (for an odd
-                        # step: of the tile that becomes "this tile" when it rotates its addresses)
-                        self.lds(("delta", k + 2, rr),
-                                 f"ds_read_b128 {self.vr(32 + 16 * par + 4 * rr, 4)}, v{self.ALD_NXT} "
-                                 f"offset:{self.row_off(par, 1, rr)}")
-                    else:
-                        g4 = rr - 4
-                        src = self.ALD_NXT if par == 1 else self.ALD_CUR
-                        self.lds(("lse", k + 1, g4),
-                                 f"ds_read_b128 {self.vr(80 + 4 * g4, 4)}, v{src} offset:{self.row_off(par ^ 1, 0, g4)}")
-                # the score accumulator of block k + 2 starts at zero (edge blocks: end of the step)
-                for op in zero[idx * nz:(idx + 1) * nz]:
-                    self.emit(op)
+                assert NB - i0 >= 4
+                if i0 <= idx < i0 + 4:
+                    for rr in range(2 * (idx - i0), 2 * (idx - i0) + 2):
+                        if rr < 4:
+                            self.lds(("lse", k + 2, rr),
+                                     f"ds_read_b128 {self.vr(16 * par + 4 * rr, 4)}, v{self.ALD_NXT} "
+                                     f"offset:{self.row_off(par, 0, rr)}")
+                        else:
+                            self.lds(("delta", k + 2, rr - 4),
+                                     f"ds_read_b128 {self.vr(32 + 16 * par + 4 * (rr - 4), 4)}, v{self.ALD_NXT} "
+                                     f"offset:{self.row_off(par, 1, rr - 4)}")
                 if par == 1:
                     n_add = -(-len(adds) // max(NB - 1, 1))
                     if idx >= 1:
@@ -305,6 +285,12 @@ class Gen:
                      f"s_cmp_le_i32 s66, s69",
                      f"s_cbranch_scc1 Lnomask_{label}",
                      f"Lmask_{label}:"]
+        # (the lse of that block has to be there; the other path does not wait and the static count
+        # of returned reads stays that of the other path)
+        if ("lse", k + 2, 3) in self.issued:
+            idx = len(self.issued) - 1 - self.issued[::-1].index(("lse", k + 2, 3))
+            if idx > self.done:
+                self.out.append(f"s_waitcnt lgkmcnt({min(len(self.issued) - 1 - idx, 15)})")
         self.out += mask
         self.out.append(f"Lnomask_{label}:")
         parts.append(self.out)
@@ -323,7 +309,7 @@ class Gen:
         return self.out
 
 
-SCALARS = ["sl2e", "qt1", "t", "q64", "n32", "st0", "st1", "st2", "wave_tile", "wave_rows", "last_row", "qlo_max",
+SCALARS = ["spare", "qt1", "t", "q64", "n32", "st0", "st1", "st2", "wave_tile", "wave_rows", "last_row", "qlo_max",
            "rq0", "rq1", "rq2", "rq3", "rg0", "rg1", "rg2", "rg3", "soff_q", "soff_g", "istep_q", "istep_g",
            "tstep_q", "tstep_g", "tmp0", "tmp1", "tmp2", "qhi_min"]          # v208 + i  ->  s40 + i
 
@@ -376,15 +362,17 @@ def generate(D, dt):
     for j in range(PF):
         p.fetch(NS + j, j, 1, True)   # same ring positions as any step's slots 0..6 (NS % RING == 0)
     for rr in range(4):
+        p.lds(("lse", 0, rr), f"ds_read_b128 {p.vr(4 * rr, 4)}, v{p.ALD_NXT} offset:{p.row_off(0, 0, rr)}")
+    for rr in range(4):
         p.lds(("delta", 0, rr), f"ds_read_b128 {p.vr(32 + 4 * rr, 4)}, v{p.ALD_NXT} offset:{p.row_off(0, 1, rr)}")
+    p.emit("s_waitcnt lgkmcnt(0)")
     p.emit("s_add_i32 s44, s43, 64")     # first row of block 0 of tile s42 + 1
     for op in p.mask_ops(0):
         p.emit(op)
+    # the phantom block: every probability exp2(-inf) = 0
     for i in range(16):
-        p.emit(f"v_mov_b32 {p.S(1, i)}, 0xff800000")
+        p.emit(f"v_mov_b32 {p.S(1, i)}, 0x7f800000")
         p.emit(f"v_mov_b32 {p.DP(1, i)}, 0")
-        p.emit(f"v_mov_b32 {p.LR(i)}, 0")
-    p.emit("s_waitcnt lgkmcnt(0)")
     issue, lpt = issue_tile(g)
     L = lambda name: f"{name}_{D}_{dt}_%="
     text = p.out
