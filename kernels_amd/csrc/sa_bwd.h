@@ -587,8 +587,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
   const int gk_last = k0 + TKB - 1 < L ? k0 + TKB - 1 : L - 1;
   const int qt0 = win_lo(k0) / TQ, qt1 = (win_hi(gk_last) + TQ - 1) / TQ;
 
-  const float sl2e = fabsf(p.scale_log2e);
-  const bool neg = p.scale_log2e < 0.0f;
+  const float kmul = -p.scale_log2e;
 
   const T* qbase = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)hd * p.q_sh;
   const T* gbase = reinterpret_cast<const T*>(p.d_o) + (int64_t)b * p.do_sb + (int64_t)hd * p.do_sh;
@@ -627,8 +626,11 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
                   (int64_t)kr * p.v_st;
 #pragma unroll
     for (int g = 0; g < NF; ++g) {
+      // K enters multiplied by -scale*log2(e), rounded to the element type: the score accumulator
+      // starts at lse and ends at lse - score*scale*log2(e), whose negated exp2 is the probability
       kf[g] = *reinterpret_cast<const Frag*>(kp + (g * 2 + h) * E::VEC);
-      if (neg) kf[g] = negate<T>(kf[g]);
+#pragma unroll
+      for (int e = 0; e < E::VEC; ++e) kf[g][e] = (T)((float)kf[g][e] * kmul);
       // V enters negated: the dP accumulator starts at delta and ends at delta - dP
       vf[g] = negate<T>(*reinterpret_cast<const Frag*>(vp + (g * 2 + h) * E::VEC));
     }
@@ -657,19 +659,16 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
 #pragma unroll
     for (int qb = 0; qb < QBN; ++qb) {
       f32x16 s[1], dp[1];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[0][i] = 0.0f;
-      // lse / delta of the 16 rows this lane holds, fetched ahead of the products; delta is
-      // read straight into the dP accumulator
-      f32x4 l4[4];
+      // lse / delta of the 16 rows this lane holds, fetched ahead of the products and read
+      // straight into the score and dP accumulators
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         const int r = qb * 32 + 8 * g4 + 4 * h;     // tile row of 4 consecutive C-fragment rows
         const float* chunk = ld_t + (r / RPW) * 2 * RPW + (r % RPW);
-        l4[g4] = *reinterpret_cast<const f32x4*>(chunk);
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(chunk);
         const f32x4 d4 = *reinterpret_cast<const f32x4*>(chunk + RPW);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dp[0][4 * g4 + e] = d4[e];
+        for (int e = 0; e < 4; ++e) s[0][4 * g4 + e] = l4[e], dp[0][4 * g4 + e] = d4[e];
       }
       // S[q][key] = Q K^T and dP[q][key] = dO V^T
       mma_rows_pair<T, D>(s[0], dp[0], Qt, Gt, qb * 32, kf, vf, lane);
@@ -678,7 +677,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int i = 4 * g4 + e;
-          const float pr = fast_exp2(__builtin_fmaf(s[0][i], sl2e, -l4[g4][e]));
+          const float pr = fast_exp2(-s[0][i]);
           s[0][i] = pr;
           dp[0][i] = pr * dp[0][i];   // = -dS
         }

@@ -226,6 +226,7 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   constexpr int TILE = TK * D;            // elements per K or V tile
   constexpr int STAGE = 2 * TILE;
   constexpr float kRescaleGap = 8.0f;
+  constexpr float kSumLimit = 256.0f;
   using Loader = AsyncTile<T, D, TK, NW>;
   constexpr int LPT = 2 * Loader::PER_WAVE;   // async loads per wave per stage (K and V)
 
@@ -363,40 +364,51 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
           for (int i = 0; i < 16; ++i) s[qb][kb][i] = keep_or_neg_inf(s[qb][kb][i], keep_bits(rm, i));
         }
       }
-      float mx = -INFINITY;
-      {
-        float mk[KBN];   // one chain per key block, so that consecutive instructions are independent
+      // Probabilities relative to the running maximum as it stands.  The maximum is only looked
+      // for when they show that it has been left behind: a tile whose probabilities of one half
+      // row add up to at most kSumLimit holds no score more than log2(kSumLimit) above it, which
+      // is harmless in fp32 and in the 16-bit operand (the result does not depend on which
+      // maximum is subtracted).  Lanes without a maximum yet always look for one.
+      float rs[2];
+      auto probabilities = [&](float m_use) {
+        rs[0] = rs[1] = 0.0f;
 #pragma unroll
-        for (int kb = 0; kb < KBN; ++kb) mk[kb] = -INFINITY;
+        for (int kb = 0; kb < KBN; ++kb) {
+          f32x16 pr;
 #pragma unroll
-        for (int i = 0; i < 16; i += 2)
+          for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(__builtin_fmaf(s[qb][kb][i], sl2e, -m_use));
+          pack_c<T>(pb[qb][kb], pr);
+          rs[0] = sum_frag(pb[qb][kb][0], rs[0]);
+          rs[1] = sum_frag(pb[qb][kb][1], rs[1]);
+        }
+      };
+      probabilities(m_run[qb] == -INFINITY ? 0.0f : m_run[qb]);
+      const bool behind = !(rs[0] + rs[1] <= kSumLimit) || m_run[qb] == -INFINITY;   // true for NaN too
+      if (__builtin_amdgcn_ballot_w64(behind) != 0) {
+        float mx = -INFINITY;
+        {
+          float mk[KBN];   // one chain per key block, so that consecutive instructions are independent
 #pragma unroll
-          for (int kb = 0; kb < KBN; ++kb) mk[kb] = fast_max3(mk[kb], s[qb][kb][i], s[qb][kb][i + 1]);
+          for (int kb = 0; kb < KBN; ++kb) mk[kb] = -INFINITY;
 #pragma unroll
-        for (int kb = 0; kb < KBN; ++kb) mx = fast_max(mx, mk[kb]);
-      }
-      mx = half_max(mx) * sl2e;
-      const bool move = mx > m_run[qb] + kRescaleGap;
-      if (__builtin_amdgcn_ballot_w64(move) != 0) {
-        const float alpha = move ? fast_exp2(m_run[qb] - mx) : 1.0f;
-        m_run[qb] = move ? mx : m_run[qb];
-        l_run[qb] *= alpha;
+          for (int i = 0; i < 16; i += 2)
 #pragma unroll
-        for (int m = 0; m < DB; ++m)
+            for (int kb = 0; kb < KBN; ++kb) mk[kb] = fast_max3(mk[kb], s[qb][kb][i], s[qb][kb][i + 1]);
 #pragma unroll
-          for (int i = 0; i < 16; ++i) oacc[qb][m][i] *= alpha;
-      }
-      const float m_use = m_run[qb] == -INFINITY ? 0.0f : m_run[qb];
+          for (int kb = 0; kb < KBN; ++kb) mx = fast_max(mx, mk[kb]);
+        }
+        mx = half_max(mx) * sl2e;
+        const bool move = mx > m_run[qb] + kRescaleGap;   // false for mx = -inf or NaN
+        if (__builtin_amdgcn_ballot_w64(move) != 0) {
+          const float alpha = move ? fast_exp2(m_run[qb] - mx) : 1.0f;
+          m_run[qb] = move ? mx : m_run[qb];
+          l_run[qb] *= alpha;
 #pragma unroll
-      for (int kb = 0; kb < KBN; ++kb)
+          for (int m = 0; m < DB; ++m)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[qb][kb][i] = fast_exp2(__builtin_fmaf(s[qb][kb][i], sl2e, -m_use));
-      float rs[2] = {0.0f, 0.0f};
-#pragma unroll
-      for (int kb = 0; kb < KBN; ++kb) {
-        pack_c<T>(pb[qb][kb], s[qb][kb]);
-        rs[0] = sum_frag(pb[qb][kb][0], rs[0]);
-        rs[1] = sum_frag(pb[qb][kb][1], rs[1]);
+            for (int i = 0; i < 16; ++i) oacc[qb][m][i] *= alpha;
+          probabilities(m_run[qb] == -INFINITY ? 0.0f : m_run[qb]);
+        }
       }
       l_run[qb] += rs[0] + rs[1];
     }
