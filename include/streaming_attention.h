@@ -148,7 +148,8 @@ int sa_query(int what);
  * (context_size * (back_contexts + 1) < 1024, < 4096, >= 4096).
  *   kernel = 0: forward   variant 0 = 4 waves (128 queries) per workgroup, 1 = 8 waves (256 queries)
  *   kernel = 1: dQ        variant 0 = 4 waves, 1 = 8 waves, 2 = software-pipelined kernel (D = 128)
- *   kernel = 2: dK/dV     variant 0 = block-skipping kernel, 1 = software-pipelined kernel (D = 128)
+ *   kernel = 2: dK/dV     variant 0 = block-skipping kernel, 1 = software-pipelined kernel (D = 128),
+ *                         2 = wave pairs (two waves per SIMD share 32 keys: one forms S and dV, the other dP and dK)
  * sa_launch_choice() returns the variant a call with these sizes runs (-1 for a D outside {64, 128},
  * a kernel id outside 0..2, context_size < 1 or back_contexts < 0).  Every variant computes the same
  * function. */

@@ -605,8 +605,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
       r = r < L ? r : L - 1;
       const float* src = (lane < RPW ? lse_base : delta_base) + r;
       float* dst = reinterpret_cast<float*>(stage_ptr(t) + 2 * TILE * sizeof(T)) + wave * 2 * RPW;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (SA_LDS void*)dst, 4, 0, 0);
+      async_copy_f32(src, dst);
     }
     ldq.issue(st, wave);
     ldg.issue(st + TILE, wave);

@@ -218,14 +218,14 @@ SA_DEV void pipeline(LoadF&& load, UseF&& use) {
 
 // acc[nb] += A_nb * B for NB row blocks of a row-major LDS tile that share the register
 // fragments bf:  acc[nb][row r][col c] += sum_k tile[row0 + nb*32 + r][k] * B[k][c].
-template <typename T, int D, int NB, int NF>
+template <typename T, int D, int NB, int NF, int GRP = 4>
 SA_DEV void mma_rows(f32x16 (&acc)[NB], const T* tile, int row0, const typename Elem<T>::Frag (&bf)[NF],
                      int lane) {
   using G_ = TileGeom<T, D>;
   static_assert(NF == G_::NF, "one register fragment per 2*VEC slice of the head dimension");
   constexpr int PITCH = G_::PITCH, VEC = Elem<T>::VEC;
   const int c = lane & 31, h = lane >> 5;
-  constexpr int N = NB * NF, G = N < 4 ? N : 4;
+  constexpr int N = NB * NF, G = N < GRP ? N : GRP;
   // row0 is a multiple of 32, so the swizzle of this lane's rows depends on c alone
   const T* base = tile + (row0 + c) * PITCH;
   const int sw = G_::swz(c);
@@ -380,7 +380,7 @@ SA_DEV void mma_tr_pair(f32x16 (&acc0)[NM], f32x16 (&acc1)[NM], const T* X0, con
 }
 
 // 16-bit only: acc[q][m] += X^T * B[q] for 32-row block rb of tile X, B[q] packed by pack_c.
-template <typename T, int D, int NQ, int NM>
+template <typename T, int D, int NQ, int NM, int GRP = 4>
 SA_DEV void mma_tr_n(f32x16 (&acc)[NQ][NM], const T* X, int rb, const typename Elem<T>::Frag (&b)[NQ][2],
                      int lane) {
   using E = Elem<T>;
@@ -393,7 +393,7 @@ SA_DEV void mma_tr_n(f32x16 (&acc)[NQ][NM], const T* X, int rb, const typename E
   const int r_lo = 4 * h + (j >> 2);
   const int col = mb + 4 * (j & 3);
   const T* blk = X + rb * 32 * PITCH;
-  constexpr int N = 2 * NM, G = N < 4 ? N : 4;
+  constexpr int N = 2 * NM, G = N < GRP ? N : GRP;
   pipeline<N, G>(
       [&](int it) {
         const int half = it / NM, m = it % NM;
@@ -432,7 +432,11 @@ template <typename T, int D, int ROWS, int NW> struct AsyncTile {
   // the last valid row, one per-lane byte offset that never changes, and a scalar byte offset
   // that carries the tile and the instruction.  No vector arithmetic per load, and rows past
   // the last valid one come back as zeros from the hardware's range check.
-  __amdgpu_buffer_rsrc_t rsrc;
+  // The copies are written as assembly: the compiler cannot tell which LDS reads a copy may
+  // overlap, so for copies it knows about it waits for ALL of them (vmcnt 0) before the first
+  // transposing LDS read that follows and before every barrier, which exposes the whole latency of
+  // the prefetch.  Completion is the caller's business anyway (wait_loads + barrier).
+  u32x4 rsrc;
   uint32_t voff;      // byte offset of this lane's 16 bytes inside instruction 0 of tile 0
   uint32_t soff;      // wave-uniform byte offset of the next tile
   uint32_t istep;     // bytes between rows of consecutive instructions of one wave
@@ -443,7 +447,11 @@ template <typename T, int D, int ROWS, int NW> struct AsyncTile {
     const int lrow = lane / G_::CPR, pch = lane % G_::CPR;
     const uint32_t rs = (uint32_t)row_stride;
     const uint32_t bytes = ((uint32_t)last_row * rs + (uint32_t)D) * ES;
-    rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gbase), 0, (int)bytes, 0x00020000);
+    const uint64_t addr = reinterpret_cast<uint64_t>(gbase);
+    rsrc[0] = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)addr);
+    rsrc[1] = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(addr >> 32) & 0xFFFFu));   // stride 0
+    rsrc[2] = (uint32_t)__builtin_amdgcn_readfirstlane((int)bytes);
+    rsrc[3] = 0x00020000u;
     voff = ((uint32_t)(wave * RPI + lrow) * rs + (uint32_t)((pch ^ G_::swz(wave * RPI + lrow)) * Elem<T>::VEC)) * ES;
     soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)first_row * rs * ES));
     istep = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(NW * RPI) * rs * ES));
@@ -455,13 +463,26 @@ template <typename T, int D, int ROWS, int NW> struct AsyncTile {
 #pragma unroll
     for (int i = I0; i < I1; ++i) {
       T* dst = tile + (i * NW + wave) * RPI * D;           // wave-uniform
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (SA_LDS void*)dst, 16, (int)voff,
-                                               (int)(soff + (uint32_t)i * istep), 0, 0);
+      const uint32_t lds_addr = (uint32_t)(uintptr_t)(SA_LDS void*)dst;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                   :
+                   : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff + (uint32_t)i * istep)
+                   : "memory", "m0");
     }
   }
   SA_DEV void issue(T* tile, int wave) const { issue_part<0, PER_WAVE>(tile, wave); }
   SA_DEV void advance() { soff += tstep; }
 };
+
+// Asynchronous copy of one float per active lane to consecutive LDS words starting at dst
+// (wave-uniform), written as assembly for the same reason as the tile copies above.
+SA_DEV void async_copy_f32(const float* src, float* dst) {
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(SA_LDS void*)dst;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+               :
+               : "s"(lds_addr), "v"(src)
+               : "memory", "m0");
+}
 
 // s_waitcnt vmcnt(N), other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
 template <int N> SA_DEV void wait_loads() {

@@ -10,6 +10,7 @@
 #include "sa_bwd.h"
 #include "sa_bwd3.h"
 #include "sa_bwd4.h"
+#include "sa_bwd_split.h"
 #endif
 
 namespace sa {
@@ -205,9 +206,32 @@ template <int D> static int dkdv3_launch(BwdParams p, hipStream_t st) {
     return SA_ERR_HEAD_DIM;
   }
 }
+// wave pairs: 8 waves (two per SIMD) own 128 keys
+template <int D> static int dkdv_split_launch(BwdParams p, hipStream_t st) {
+  using C = Cfg<ElemT>;
+  if constexpr (C::fwd2(D)) {
+    constexpr int TKB = 128, TQ = 64, NST = 3, NW = 8;
+    // tile stages followed by the pairs' exchange slots; the epilogue's row patches reuse the stages
+    constexpr size_t stages = (size_t)NST * (2 * TQ * D * sizeof(ElemT) + 2 * TQ * sizeof(float));
+    constexpr size_t patches = (size_t)NW * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
+    static_assert(patches <= stages, "row patches must not reach the exchange slots");
+    constexpr size_t lds = stages + (size_t)4 * 2 * 2048;
+    auto kern = dkdv_split_kernel<ElemT, D, NST>;
+    static PrepareState once;
+    if (int rc = prepare(kern, lds, once)) return rc;
+    p.n_tiles = (int)ceil_div(p.T, TKB);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+  } else {
+    return SA_ERR_HEAD_DIM;
+  }
+}
 template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
+    if (launch_choice(D, p.C, p.R).dkdv == DKDV_SPLIT) return dkdv_split_launch<D>(p, st);
     // The pipelined kernel (head dimension 128) makes every wave walk the whole window of its
     // workgroup's 128 keys; that wastes nothing once a chunk holds at least those 128 keys.  Smaller
     // chunks go to the kernel whose waves skip the query tiles outside their own 32 keys' windows.

@@ -52,7 +52,8 @@ enum DqVariant : int { DQ_NARROW = 0, DQ_WIDE = 1,
                        DQ_VARIANTS = 3 };
 enum DkdvVariant : int { DKDV_BLOCKSKIP = 0,   // every wave skips the query tiles outside its own 32 keys' windows
                          DKDV_PIPELINED = 1,   // hand-scheduled loop, head dimension 128 only
-                         DKDV_VARIANTS = 2 };
+                         DKDV_SPLIT = 2,       // wave pairs share 32 keys: one wave forms S and dV, the other dP and dK
+                         DKDV_VARIANTS = 3 };
 struct LaunchChoice { int fwd, dq, dkdv; };
 constexpr int TUNE_CHUNK_CLASSES = 7;    // context_size < 32, < 64, < 128, < 256, < 512, < 1024, >= 1024
 constexpr int TUNE_WINDOW_CLASSES = 3;   // context_size * (back_contexts + 1) < 1024, < 4096, >= 4096
@@ -71,7 +72,7 @@ inline LaunchChoice launch_choice(int D, int chunk, int back) {
   if (g_tune_override[0] >= 0 && g_tune_override[0] < FWD_VARIANTS) c.fwd = g_tune_override[0];
   if (g_tune_override[1] >= 0 && g_tune_override[1] < DQ_VARIANTS) c.dq = g_tune_override[1];
   if (g_tune_override[2] >= 0 && g_tune_override[2] < DKDV_VARIANTS) c.dkdv = g_tune_override[2];
-  if (D != 128) c.dkdv = DKDV_BLOCKSKIP;
+  if (D != 128 && c.dkdv == DKDV_PIPELINED) c.dkdv = DKDV_BLOCKSKIP;
   if (D != 128 && c.dq == DQ_PIPELINED) c.dq = DQ_NARROW;
   return c;
 }

@@ -19,9 +19,12 @@ _HEAD_DIMS = (16, 32, 64, 128, 256)
 _VEC_BYTES = 16
 
 
+_DTYPE_IDS = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}   # SA_DTYPE_* of the C ABI
+
+
 def _dtype_id(dtype: torch.dtype) -> int:
     try:
-        return _lib.DTYPE_IDS[str(dtype)]
+        return _DTYPE_IDS[dtype]
     except KeyError:
         raise AssertionError(f"unsupported dtype {dtype}: expected float32, float16 or bfloat16") from None
 
@@ -55,7 +58,9 @@ def _lens_args(lens: Optional[torch.Tensor]):
 
 
 def _stream(device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Handle of torch's current stream on ``device`` (what ``current_stream(device).cuda_stream``
+    returns, without building the Stream object)."""
+    return torch._C._cuda_getCurrentRawStream(device.index)
 
 
 class _on_device:
@@ -65,8 +70,7 @@ class _on_device:
     __slots__ = ("ctx",)
 
     def __init__(self, device):
-        idx = device.index
-        self.ctx = None if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(device)
+        self.ctx = None if device.index == torch._C._cuda_getDevice() else torch.cuda.device(device)
 
     def __enter__(self):
         if self.ctx is not None:
@@ -93,20 +97,43 @@ def _validate_placement(q, k, v, lens, *others):
 
 def _validate(q, k, v, lens, context_size, back_contexts, sm_scale, *others):
     # same conditions, same exception type as kernel.py:1288-1295
-    _validate_placement(q, k, v, lens, *others)
-    batch, _, T, head_dim = q.shape
+    shape, dev = q.shape, q.device
+    plain = (len(shape) == 4 and k.shape == shape and v.shape == shape
+             and k.device == dev and v.device == dev and (lens is None or lens.device == dev))
+    for t in others:
+        plain = plain and t.shape == shape and t.device == dev
+    if not plain:   # name the condition that failed
+        _validate_placement(q, k, v, lens, *others)
+    batch, _, T, head_dim = shape
     assert back_contexts >= 0 and context_size >= 1
     assert head_dim in _HEAD_DIMS
     assert head_dim == k.shape[-1] and head_dim == v.shape[-1]
     assert T == k.shape[-2] and T == v.shape[-2]
     assert sm_scale is not None
-    assert lens is None or (lens.dtype == torch.int32 and batch == len(lens) and lens.ndim == 1)
+    assert lens is None or (lens.dtype == torch.int32 and lens.ndim == 1 and batch == lens.shape[0])
     assert q.dtype == k.dtype == v.dtype
 
 
-@torch.library.custom_op(
-    "alexdremov_streaming_attention::forward", mutates_args=(), device_types=("cuda",)
+# The two ops are declared with the same schemas that the reference's ``torch.library.custom_op``
+# decorators infer (kernel.py:1270-1284, 1360-1376) and carry the pt2-compliance tag that the
+# decorator sets, but through ``torch.library.Library``: a call then goes from the dispatcher
+# straight to the functions below, without the per-call Python wrappers of ``custom_op`` and of
+# ``register_autograd``, which cost more host time per step than all four kernels of a small problem
+# take on the GPU.
+_LIBRARY = torch.library.Library("alexdremov_streaming_attention", "DEF")
+_LIBRARY.define(
+    "forward(Tensor q, Tensor k, Tensor v, Tensor? lens, SymInt context_size, SymInt back_contexts, "
+    "float sm_scale, bool autotune, bool return_lse, bool prescale_qk, str precision) -> (Tensor, Tensor)",
+    tags=(torch.Tag.pt2_compliant_tag,),
 )
+_LIBRARY.define(
+    "backward(Tensor q, Tensor k, Tensor v, Tensor? lens, Tensor o, Tensor lse, Tensor do, "
+    "SymInt context_size, SymInt back_contexts, float sm_scale, bool autotune, bool prescale_qk, "
+    "str precision) -> (Tensor, Tensor, Tensor)",
+    tags=(torch.Tag.pt2_compliant_tag,),
+)
+
+
 def attention_forward_adapter(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -124,7 +151,7 @@ def attention_forward_adapter(
     B, H, T, D = q.shape
     lib = _lib.load()
     # the kernel writes every element (zeros at padded positions included)
-    O = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    O = torch.empty_like(q, memory_format=torch.contiguous_format)
     LSE = torch.empty((B, H, T), dtype=torch.float32, device=q.device) if return_lse else None
     if q.numel() > 0:
         qk, kk, vk = _kernel_layout(q), _kernel_layout(k), _kernel_layout(v)
@@ -143,7 +170,10 @@ def attention_forward_adapter(
     return O, LSE
 
 
-@torch.library.register_fake("alexdremov_streaming_attention::forward")
+_LIBRARY.impl("forward", attention_forward_adapter, "CUDA")
+
+
+@torch.library.register_fake("alexdremov_streaming_attention::forward", lib=_LIBRARY)
 def attention_forward_adapter_abstract(
     q, k, v, lens, context_size, back_contexts, sm_scale, autotune, return_lse, prescale_qk, precision
 ):
@@ -153,9 +183,6 @@ def attention_forward_adapter_abstract(
     )
 
 
-@torch.library.custom_op(
-    "alexdremov_streaming_attention::backward", mutates_args=(), device_types=("cuda",)
-)
 def attention_backward_adapter(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -174,9 +201,9 @@ def attention_backward_adapter(
     _validate(q, k, v, lens, context_size, back_contexts, sm_scale, o, do)
     B, H, T, D = q.shape
     lib = _lib.load()
-    DQ = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    DK = torch.empty(k.shape, dtype=k.dtype, device=k.device)
-    DV = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+    DQ = torch.empty_like(q, memory_format=torch.contiguous_format)
+    DK = torch.empty_like(k, memory_format=torch.contiguous_format)
+    DV = torch.empty_like(v, memory_format=torch.contiguous_format)
     if q.numel() == 0:
         return DQ, DK, DV
     qk, kk, vk = _kernel_layout(q), _kernel_layout(k), _kernel_layout(v)
@@ -216,7 +243,10 @@ def attention_backward_adapter(
     return DQ, DK, DV
 
 
-@torch.library.register_fake("alexdremov_streaming_attention::backward")
+_LIBRARY.impl("backward", attention_backward_adapter, "CUDA")
+
+
+@torch.library.register_fake("alexdremov_streaming_attention::backward", lib=_LIBRARY)
 def attention_backward_adapter_abstract(
     q, k, v, lens, o, lse, do, context_size, back_contexts, sm_scale, autotune, prescale_qk, precision
 ):
@@ -227,29 +257,33 @@ def attention_backward_adapter_abstract(
     )
 
 
-def _setup_context(ctx, inputs, output):
-    O, LSE = output
-    (q, k, v, lens, context_size, back_contexts, sm_scale, autotune, return_lse, prescale_qk, precision) = inputs
-    ctx.save_for_backward(q, k, v, O, LSE, lens)
-    ctx.context_size = context_size
-    ctx.back_contexts = back_contexts
-    ctx.autotune = autotune
-    ctx.sm_scale = sm_scale
-    ctx.prescale_qk = prescale_qk
-    ctx.precision = precision
+class _StreamingAttention(torch.autograd.Function):
+    """Autograd glue of the forward op (kernel.py:1467-1530): saves q, k, v, O, LSE and lens, hands
+    dO to the backward op, lets no gradient flow through the log-sum-exp output (kernel.py:1498)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, lens, context_size, back_contexts, sm_scale, autotune, return_lse,
+                prescale_qk, precision):
+        with torch._C._AutoDispatchBelowAutograd():
+            O, LSE = torch.ops.alexdremov_streaming_attention.forward(
+                q, k, v, lens, context_size, back_contexts, sm_scale, autotune, return_lse, prescale_qk, precision)
+        ctx.save_for_backward(q, k, v, O, LSE, lens)
+        ctx.context_size = context_size
+        ctx.back_contexts = back_contexts
+        ctx.autotune = autotune
+        ctx.sm_scale = sm_scale
+        ctx.prescale_qk = prescale_qk
+        ctx.precision = precision
+        ctx.mark_non_differentiable(LSE)
+        return O, LSE
+
+    @staticmethod
+    def backward(ctx, do, dlse):
+        q, k, v, o, lse, lens = ctx.saved_tensors
+        DQ, DK, DV = torch.ops.alexdremov_streaming_attention.backward(
+            q, k, v, lens, o, lse, do, ctx.context_size, ctx.back_contexts, ctx.sm_scale,
+            ctx.autotune, ctx.prescale_qk, ctx.precision)
+        return DQ, DK, DV, None, None, None, None, None, None, None, None
 
 
-def _backward(ctx, do, dlse):
-    # no gradient flows through the log-sum-exp output (kernel.py:1498)
-    q, k, v, o, lse, lens = ctx.saved_tensors
-    DQ, DK, DV = torch.ops.alexdremov_streaming_attention.backward(
-        q=q, k=k, v=v, lens=lens, o=o, lse=lse, do=do,
-        context_size=ctx.context_size, back_contexts=ctx.back_contexts, sm_scale=ctx.sm_scale,
-        autotune=ctx.autotune, prescale_qk=ctx.prescale_qk, precision=ctx.precision,
-    )
-    return DQ, DK, DV, None, None, None, None, None, None, None, None
-
-
-torch.library.register_autograd(
-    "alexdremov_streaming_attention::forward", _backward, setup_context=_setup_context
-)
+_LIBRARY.impl("forward", _StreamingAttention.apply, "Autograd")

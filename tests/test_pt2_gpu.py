@@ -43,7 +43,7 @@ def test_opcheck(dtype, use_lens):
 
 @pytest.mark.parametrize("lens_mode", ["none", "random"])
 def test_compiled_wrapper_does_not_recompile_per_shape(lens_mode, monkeypatch):
-    monkeypatch.delenv("STREAMING_ATTENTION_EAGER", raising=False)
+    monkeypatch.setenv("STREAMING_ATTENTION_COMPILED", "1")
     from streaming_attention import streaming_attention
 
     torch._dynamo.reset()
@@ -65,7 +65,7 @@ def test_compiled_wrapper_does_not_recompile_per_shape(lens_mode, monkeypatch):
 
 
 def test_inside_a_compiled_function(monkeypatch):
-    monkeypatch.delenv("STREAMING_ATTENTION_EAGER", raising=False)
+    monkeypatch.setenv("STREAMING_ATTENTION_COMPILED", "1")
     from oracle import sa_oracle
     from streaming_attention import streaming_attention
     from tests.helpers import assert_close
