@@ -41,7 +41,7 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
   constexpr int STAGE_BYTES = 2 * TILE * (int)sizeof(T) + 2 * TQ * (int)sizeof(float);
   constexpr int XSLOT = 64 * 2 * 16;             // bytes of one exchange slot: two fragments per lane
   constexpr int XBUF_OFF = NST * STAGE_BYTES;    // exchange slots follow the stages: [pair][2][XSLOT]
-  using Loader = AsyncTile<T, D, TQ, NW>;
+  using Loader = AsyncTile<T, D, TQ, NW, true>;   // copies as assembly: three stages, see AsyncTile
   constexpr int LPT = 2 * Loader::PER_WAVE + 1;  // asynchronous loads per wave per tile
 #ifndef SA_SPLIT_GRP
 #define SA_SPLIT_GRP 2
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
       r = r < L ? r : L - 1;
       const float* src = (lane < RPW ? lse_base : delta_base) + r;
       float* dst = reinterpret_cast<float*>(smem_raw + stage_off + 2 * TILE * sizeof(T)) + wave * 2 * RPW;
-      async_copy_f32(src, dst);
+      async_copy_f32<true>(src, dst);
     }
     ldq.issue(st, wave);
     ldg.issue(st + TILE, wave);

@@ -418,7 +418,7 @@ SA_DEV void mma_tr_n(f32x16 (&acc)[NQ][NM], const T* X, int rb, const typename E
 //
 // Tiles are issued in ascending order.  Offsets are 32-bit byte offsets inside one (batch, head)
 // slice: the host checks that T * row_stride * sizeof(T) fits.
-template <typename T, int D, int ROWS, int NW> struct AsyncTile {
+template <typename T, int D, int ROWS, int NW, bool ASM_COPIES = false> struct AsyncTile {
   using G_ = TileGeom<T, D>;
   static_assert(G_::SWZ, "asynchronous tiles use the swizzled layout");
   static constexpr int ROW_BYTES = D * (int)sizeof(T);
@@ -432,11 +432,13 @@ template <typename T, int D, int ROWS, int NW> struct AsyncTile {
   // the last valid row, one per-lane byte offset that never changes, and a scalar byte offset
   // that carries the tile and the instruction.  No vector arithmetic per load, and rows past
   // the last valid one come back as zeros from the hardware's range check.
-  // The copies are written as assembly: the compiler cannot tell which LDS reads a copy may
-  // overlap, so for copies it knows about it waits for ALL of them (vmcnt 0) before the first
-  // transposing LDS read that follows and before every barrier, which exposes the whole latency of
-  // the prefetch.  Completion is the caller's business anyway (wait_loads + barrier).
-  u32x4 rsrc;
+  // With ASM_COPIES the copies are written as assembly: the compiler cannot tell which LDS reads a
+  // copy may overlap, so for copies it knows about it waits for ALL of them (vmcnt 0) before the
+  // first transposing LDS read that follows and before every barrier.  A ring of two stages loses
+  // nothing by that (measured), a ring of three would lose its point.  Completion is the caller's
+  // business either way (wait_loads + barrier).
+  u32x4 rsrc;                      // descriptor words for the assembly form
+  __amdgpu_buffer_rsrc_t brsrc;    // the same descriptor for the builtin
   uint32_t voff;      // byte offset of this lane's 16 bytes inside instruction 0 of tile 0
   uint32_t soff;      // wave-uniform byte offset of the next tile
   uint32_t istep;     // bytes between rows of consecutive instructions of one wave
@@ -452,6 +454,7 @@ template <typename T, int D, int ROWS, int NW> struct AsyncTile {
     rsrc[1] = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(addr >> 32) & 0xFFFFu));   // stride 0
     rsrc[2] = (uint32_t)__builtin_amdgcn_readfirstlane((int)bytes);
     rsrc[3] = 0x00020000u;
+    brsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gbase), 0, (int)bytes, 0x00020000);
     voff = ((uint32_t)(wave * RPI + lrow) * rs + (uint32_t)((pch ^ G_::swz(wave * RPI + lrow)) * Elem<T>::VEC)) * ES;
     soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)first_row * rs * ES));
     istep = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(NW * RPI) * rs * ES));
@@ -463,11 +466,18 @@ template <typename T, int D, int ROWS, int NW> struct AsyncTile {
 #pragma unroll
     for (int i = I0; i < I1; ++i) {
       T* dst = tile + (i * NW + wave) * RPI * D;           // wave-uniform
-      const uint32_t lds_addr = (uint32_t)(uintptr_t)(SA_LDS void*)dst;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                   :
-                   : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff + (uint32_t)i * istep)
-                   : "memory", "m0");
+      if constexpr (ASM_COPIES) {
+        // both scalars are wave-uniform by construction; readfirstlane makes that known to the compiler
+        const uint32_t lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(SA_LDS void*)dst);
+        const uint32_t so = (uint32_t)__builtin_amdgcn_readfirstlane((int)(soff + (uint32_t)i * istep));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(so)
+                     : "memory", "m0");
+      } else {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(brsrc, (SA_LDS void*)dst, 16, (int)voff,
+                                                 (int)(soff + (uint32_t)i * istep), 0, 0);
+      }
     }
   }
   SA_DEV void issue(T* tile, int wave) const { issue_part<0, PER_WAVE>(tile, wave); }
@@ -475,13 +485,17 @@ template <typename T, int D, int ROWS, int NW> struct AsyncTile {
 };
 
 // Asynchronous copy of one float per active lane to consecutive LDS words starting at dst
-// (wave-uniform), written as assembly for the same reason as the tile copies above.
-SA_DEV void async_copy_f32(const float* src, float* dst) {
-  const uint32_t lds_addr = (uint32_t)(uintptr_t)(SA_LDS void*)dst;
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
-               :
-               : "s"(lds_addr), "v"(src)
-               : "memory", "m0");
+// (wave-uniform); as assembly for the same reason as the tile copies above when ASM_COPIES is set.
+template <bool ASM_COPIES = false> SA_DEV void async_copy_f32(const float* src, float* dst) {
+  if constexpr (ASM_COPIES) {
+    const uint32_t lds_addr = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(SA_LDS void*)dst);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                 :
+                 : "s"(lds_addr), "v"(src)
+                 : "memory", "m0");
+  } else {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src, (SA_LDS void*)dst, 4, 0, 0);
+  }
 }
 
 // s_waitcnt vmcnt(N), other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and 15:14).
