@@ -303,10 +303,12 @@ def tune_sweep(device, iters=10):
         for dtype_name in ("bfloat16", "float16"):
             for D in (64, 128):
                 for C in (16, 32, 64, 128, 256, 512, 1024):
-                    for window in (512, 2048, 8192):   # one per window class of the table
+                    seen = set()
+                    for window in (128, 512, 2048, 8192):   # one per window class of the table
                         R = max(0, window // C - 1)
-                        if dtype_name == "float16" and window != 2048:
-                            continue   # the second type only confirms the first
+                        if R in seen or (dtype_name == "float16" and window != 2048):
+                            continue   # same problem again / the second type only confirms the first
+                        seen.add(R)
                         g = torch.Generator(device=device).manual_seed(20)
                         dt = getattr(torch, dtype_name)
                         q, k, v, d_o = [torch.randn(B, H, T, D, generator=g, device=device, dtype=torch.float32).to(dt)

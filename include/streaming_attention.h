@@ -145,7 +145,7 @@ int sa_query(int what);
  * 1154-1193, 1212-1267): the reference searches block shapes at run time, this library ships the
  * outcome of an offline sweep on MI355X, indexed by head dimension, context_size class
  * (< 32, < 64, < 128, < 256, < 512, < 1024, >= 1024) and window class
- * (context_size * (back_contexts + 1) < 1024, < 4096, >= 4096).
+ * (context_size * (back_contexts + 1) < 256, < 1024, < 4096, >= 4096).
  *   kernel = 0: forward   variant 0 = 4 waves (128 queries) per workgroup, 1 = 8 waves (256 queries)
  *   kernel = 1: dQ        variant 0 = 4 waves, 1 = 8 waves, 2 = software-pipelined kernel (D = 128)
  *   kernel = 2: dK/dV     variant 0 = block-skipping kernel, 1 = software-pipelined kernel (D = 128),

@@ -491,10 +491,13 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
     const T* Vt = Kt + TILE;
     const int k0 = t * TK;
     if (k0 + TK <= lo_min || k0 >= hi_max) continue;   // outside this wave's windows
-    const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
 
 #pragma unroll
     for (int kb = 0; kb < KBN; ++kb) {
+      // the same two tests per 32-key block: short windows end inside a tile
+      const int kb0 = k0 + kb * 32;
+      if (kb0 + 32 <= lo_min || kb0 >= hi_max) continue;
+      const bool interior = (kb0 >= lo_max) && (kb0 + 32 <= hi_min);
       f32x16 s[1], dp[1];
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[0][i] = 0.0f;
@@ -653,10 +656,13 @@ __global__ __launch_bounds__(NW * 64) void dkdv2_kernel(const BwdParams p) {
     const float* ld_t = reinterpret_cast<const float*>(stage_ptr(t) + 2 * TILE * sizeof(T));
     const int qs = t * TQ;
     if (qs + TQ <= qlo_min || qs >= qhi_max) continue;   // outside this wave's windows
-    const bool interior = (qs >= qlo_max) && (qs + TQ <= qhi_min);
 
 #pragma unroll
     for (int qb = 0; qb < QBN; ++qb) {
+      // the same two tests per 32-query block: short windows end inside a tile
+      const int qb0 = qs + qb * 32;
+      if (qb0 + 32 <= qlo_min || qb0 >= qhi_max) continue;
+      const bool interior = (qb0 >= qlo_max) && (qb0 + 32 <= qhi_min);
       f32x16 s[1], dp[1];
       // lse / delta of the 16 rows this lane holds, fetched ahead of the products and read
       // straight into the score and dP accumulators

@@ -349,16 +349,44 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
       for (int kb = 0; kb < KBN; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[qb][kb][i] = 0.0f;
-    mma_rows_n<T, D>(s, Kt, 0, qf, lane);
+    // Short windows end inside a tile: a 32-key block that no query of this wave can see is left
+    // out of both products and of the arithmetic, one that every query sees in full needs no mask.
+    bool live[KBN], inside[KBN], all_live = true;
+#pragma unroll
+    for (int kb = 0; kb < KBN; ++kb) {
+      const int kb0 = k0 + kb * 32;
+      live[kb] = kb0 + 32 > lo_min && kb0 < hi_max;
+      inside[kb] = kb0 >= lo_max && kb0 + 32 <= hi_min;
+      all_live = all_live && live[kb];
+    }
+    if (all_live) {
+      mma_rows_n<T, D>(s, Kt, 0, qf, lane);
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < KBN; ++kb) {
+        if (live[kb]) {
+          f32x16 one[QB][1];
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) one[qb][0] = s[qb][kb];
+          mma_rows_n<T, D>(one, Kt, kb * 32, qf, lane);
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb) s[qb][kb] = one[qb][0];
+        } else {
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[qb][kb][i] = -INFINITY;
+        }
+      }
+    }
 
-    const bool interior = (k0 >= lo_max) && (k0 + TK <= hi_min);
     Frag pb[QB][KBN][2];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
-      if (!interior) {
-        // keys outside [lo, hi) score -inf (whatever the product gave, NaN from padding included)
+      // keys outside [lo, hi) score -inf (whatever the product gave, NaN from padding included)
 #pragma unroll
-        for (int kb = 0; kb < KBN; ++kb) {
+      for (int kb = 0; kb < KBN; ++kb) {
+        if (live[kb] && !inside[kb]) {
           const uint32_t rm = row_mask(lo[qb] - (k0 + kb * 32), hi[qb] - (k0 + kb * 32), h);
 #pragma unroll
           for (int i = 0; i < 16; ++i) s[qb][kb][i] = keep_or_neg_inf(s[qb][kb][i], keep_bits(rm, i));
@@ -374,6 +402,7 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
         rs[0] = rs[1] = 0.0f;
 #pragma unroll
         for (int kb = 0; kb < KBN; ++kb) {
+          if (!live[kb]) continue;   // never multiplied
           f32x16 pr;
 #pragma unroll
           for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(__builtin_fmaf(s[qb][kb][i], sl2e, -m_use));
@@ -382,9 +411,16 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
           rs[1] = sum_frag(pb[qb][kb][1], rs[1]);
         }
       };
-      probabilities(m_run[qb] == -INFINITY ? 0.0f : m_run[qb]);
-      const bool behind = !(rs[0] + rs[1] <= kSumLimit) || m_run[qb] == -INFINITY;   // true for NaN too
-      if (__builtin_amdgcn_ballot_w64(behind) != 0) {
+      // A wave none of whose lanes has a maximum yet (its first visible tile) goes straight to the
+      // search: the speculative pass would be thrown away, and short windows are all first tiles.
+      const bool fresh = __builtin_amdgcn_ballot_w64(m_run[qb] != -INFINITY) == 0;
+      bool search = fresh;
+      if (!fresh) {
+        probabilities(m_run[qb] == -INFINITY ? 0.0f : m_run[qb]);
+        const bool behind = !(rs[0] + rs[1] <= kSumLimit) || m_run[qb] == -INFINITY;   // true for NaN too
+        search = __builtin_amdgcn_ballot_w64(behind) != 0;
+      }
+      if (search) {
         float mx = -INFINITY;
         {
           float mk[KBN];   // one chain per key block, so that consecutive instructions are independent
@@ -399,14 +435,16 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
         }
         mx = half_max(mx) * sl2e;
         const bool move = mx > m_run[qb] + kRescaleGap;   // false for mx = -inf or NaN
-        if (__builtin_amdgcn_ballot_w64(move) != 0) {
+        if (fresh || __builtin_amdgcn_ballot_w64(move) != 0) {
           const float alpha = move ? fast_exp2(m_run[qb] - mx) : 1.0f;
           m_run[qb] = move ? mx : m_run[qb];
           l_run[qb] *= alpha;
+          if (!fresh) {   // a fresh wave has accumulated nothing yet
 #pragma unroll
-          for (int m = 0; m < DB; ++m)
+            for (int m = 0; m < DB; ++m)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) oacc[qb][m][i] *= alpha;
+              for (int i = 0; i < 16; ++i) oacc[qb][m][i] *= alpha;
+          }
           probabilities(m_run[qb] == -INFINITY ? 0.0f : m_run[qb]);
         }
       }
@@ -416,6 +454,7 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
     // O^T[d][q] += V^T P^T
 #pragma unroll
     for (int kb = 0; kb < KBN; ++kb) {
+      if (!live[kb]) continue;
       Frag bq[QB][2];
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) bq[qb][0] = pb[qb][kb][0], bq[qb][1] = pb[qb][kb][1];

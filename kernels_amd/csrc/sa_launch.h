@@ -56,13 +56,13 @@ enum DkdvVariant : int { DKDV_BLOCKSKIP = 0,   // every wave skips the query til
                          DKDV_VARIANTS = 3 };
 struct LaunchChoice { int fwd, dq, dkdv; };
 constexpr int TUNE_CHUNK_CLASSES = 7;    // context_size < 32, < 64, < 128, < 256, < 512, < 1024, >= 1024
-constexpr int TUNE_WINDOW_CLASSES = 3;   // context_size * (back_contexts + 1) < 1024, < 4096, >= 4096
+constexpr int TUNE_WINDOW_CLASSES = 4;   // context_size * (back_contexts + 1) < 256, < 1024, < 4096, >= 4096
 constexpr int chunk_class(int chunk) {
   return chunk < 32 ? 0 : chunk < 64 ? 1 : chunk < 128 ? 2 : chunk < 256 ? 3 : chunk < 512 ? 4 : chunk < 1024 ? 5 : 6;
 }
 constexpr int window_class(int chunk, int back) {
   const long long w = (long long)chunk * ((long long)back + 1);
-  return w < 1024 ? 0 : w < 4096 ? 1 : 2;
+  return w < 256 ? 0 : w < 1024 ? 1 : w < 4096 ? 2 : 3;
 }
 #include "sa_tune_table.inc"
 // Variants pinned through sa_tune_override() for measurements; -1 = use the table.

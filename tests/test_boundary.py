@@ -46,14 +46,14 @@ def test_query_and_error_strings(lib):
     assert lib.sa_query(99) == -1
     assert b"success" in lib.sa_error_string(0)
     assert lib.sa_query(10) == 1 << 21
-    assert lib.sa_query(11) == 3 and lib.sa_query(12) == -1
+    assert lib.sa_query(11) == 4 and lib.sa_query(12) == -1
     # the launch-configuration table answers without a GPU and rejects what it does not cover
     for D in (64, 128):
         for C in (1, 31, 32, 100, 256, 5000):
             for R in (0, 3, 100, 2 ** 31 - 1):
                 assert lib.sa_launch_choice(D, C, R, 0) in (0, 1)
                 assert lib.sa_launch_choice(D, C, R, 1) in ((0, 1, 2) if D == 128 else (0, 1))
-                assert lib.sa_launch_choice(D, C, R, 2) in ((0, 1) if D == 128 else (0,))
+                assert lib.sa_launch_choice(D, C, R, 2) in ((0, 1, 2) if D == 128 else (0, 2))
     assert lib.sa_launch_choice(32, 64, 1, 0) == -1 and lib.sa_launch_choice(128, 0, 1, 0) == -1
     assert lib.sa_launch_choice(128, 64, 1, 3) == -1 and lib.sa_launch_choice(128, 64, -1, 0) == -1
     assert lib.sa_tune_override(0, 2) == -3 and lib.sa_tune_override(3, 0) == -3

@@ -131,10 +131,10 @@ def test_tile_edges_16bit(T, C, R, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
 @pytest.mark.parametrize("D", [64, 128])
-@pytest.mark.parametrize("C,R", [(16, 2), (48, 30), (100, 3), (200, 1), (300, 4), (600, 0), (1100, 1)])
+@pytest.mark.parametrize("C,R", [(16, 2), (20, 300), (48, 30), (100, 3), (200, 0), (200, 1), (300, 4), (600, 0), (1100, 1)])
 def test_every_table_class_16bit(C, R, D, dtype):
-    """One context_size per class of the launch-configuration table, windows in all three window
-    classes, run with the variants the table picks."""
+    """One context_size per class of the launch-configuration table, windows in all four window
+    classes (48 ... 6020 keys), run with the variants the table picks."""
     B, H, T = 2, 2, 1500
     q, k, v, d_o = make_inputs(B, H, T, D, seed=31, dtype=dtype)
     lens = torch.tensor([T, T - 333], dtype=torch.int32)
