@@ -215,7 +215,11 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
 // are 8-byte LDS reads and would otherwise cap the second product well below the MFMA
 // rate); K and V tiles are brought in by asynchronous global->LDS copies into a ring of NST
 // stages, NST-1 tiles ahead of the compute, with one barrier per key tile.
-template <typename T, int D, int QB, int NW, int TK, int NST>
+// SHORT selects the form for short windows (a handful of key tiles per workgroup): work is skipped
+// and masks are decided per 32-key block instead of per tile, and a wave's first tile goes straight
+// to the search for its maximum.  Long windows run the plain form, whose loop is a few per cent
+// tighter (fewer registers, no per-block tests).
+template <typename T, int D, int QB, int NW, int TK, int NST, bool SHORT>
 __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   using E = Elem<T>;
   using G = TileGeom<T, D>;
@@ -354,9 +358,9 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
     bool live[KBN], inside[KBN], all_live = true;
 #pragma unroll
     for (int kb = 0; kb < KBN; ++kb) {
-      const int kb0 = k0 + kb * 32;
-      live[kb] = kb0 + 32 > lo_min && kb0 < hi_max;
-      inside[kb] = kb0 >= lo_max && kb0 + 32 <= hi_min;
+      const int kb0 = SHORT ? k0 + kb * 32 : k0, kbn = SHORT ? 32 : TK;   // the block, or the whole tile
+      live[kb] = !SHORT || (kb0 + kbn > lo_min && kb0 < hi_max);
+      inside[kb] = kb0 >= lo_max && kb0 + kbn <= hi_min;
       all_live = all_live && live[kb];
     }
     if (all_live) {
@@ -413,7 +417,7 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
       };
       // A wave none of whose lanes has a maximum yet (its first visible tile) goes straight to the
       // search: the speculative pass would be thrown away, and short windows are all first tiles.
-      const bool fresh = __builtin_amdgcn_ballot_w64(m_run[qb] != -INFINITY) == 0;
+      const bool fresh = SHORT && __builtin_amdgcn_ballot_w64(m_run[qb] != -INFINITY) == 0;
       bool search = fresh;
       if (!fresh) {
         probabilities(m_run[qb] == -INFINITY ? 0.0f : m_run[qb]);

@@ -72,14 +72,14 @@ static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 #endif
 
 #if SA_KIND == 0
-template <int D, int NW> static int fwd2_launch(FwdParams p, hipStream_t st) {
+template <int D, int NW, bool SHORT> static int fwd2_launch(FwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   constexpr int TQ = NW * C::FWD2_QB * 32;
   // tile stages; the epilogue's row patches (one per wave) reuse the same memory
   constexpr size_t stages = (size_t)C::FWD2_NST * 2 * C::FWD_TK * D * sizeof(ElemT);
   constexpr size_t patches = (size_t)NW * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
   constexpr size_t lds = stages > patches ? stages : patches;
-  auto kern = fwd2_kernel<ElemT, D, C::FWD2_QB, NW, C::FWD_TK, C::FWD2_NST>;
+  auto kern = fwd2_kernel<ElemT, D, C::FWD2_QB, NW, C::FWD_TK, C::FWD2_NST, SHORT>;
   static PrepareState once;
   if (int rc = prepare(kern, lds, once)) return rc;
   p.n_tiles = (int)ceil_div(p.T, TQ);
@@ -91,8 +91,11 @@ template <int D, int NW> static int fwd2_launch(FwdParams p, hipStream_t st) {
 template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
-    return launch_choice(D, p.C, p.R).fwd == FWD_WIDE ? fwd2_launch<D, C::WIDE_NW>(p, st)
-                                                      : fwd2_launch<D, C::NARROW_NW>(p, st);
+    // windows of less than 1024 keys (the table's first two window classes) run the short-window form
+    const bool wide = launch_choice(D, p.C, p.R).fwd == FWD_WIDE;
+    if (window_class(p.C, p.R) <= 1)
+      return wide ? fwd2_launch<D, C::WIDE_NW, true>(p, st) : fwd2_launch<D, C::NARROW_NW, true>(p, st);
+    return wide ? fwd2_launch<D, C::WIDE_NW, false>(p, st) : fwd2_launch<D, C::NARROW_NW, false>(p, st);
   } else {
     constexpr int TQ = C::NW * 32;
     constexpr size_t lds = (size_t)2 * 2 * C::FWD_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
