@@ -43,10 +43,9 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
   constexpr int XBUF_OFF = NST * STAGE_BYTES;    // exchange slots follow the stages: [pair][2][XSLOT]
   using Loader = AsyncTile<T, D, TQ, NW, true>;   // copies as assembly: three stages, see AsyncTile
   constexpr int LPT = 2 * Loader::PER_WAVE + 1;  // asynchronous loads per wave per tile
-#ifndef SA_SPLIT_GRP
-#define SA_SPLIT_GRP 2
-#endif
-  constexpr int GRP = SA_SPLIT_GRP;              // LDS fragments requested ahead of the MFMAs that consume them
+  // LDS fragments requested ahead of the MFMAs that consume them: with two waves per SIMD a depth of
+  // 2 measured the same as 4 and 8 and leaves the most registers
+  constexpr int GRP = 2;
 
   extern __shared__ __attribute__((aligned(16))) char smem_raw[];
 

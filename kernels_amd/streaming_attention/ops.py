@@ -57,10 +57,16 @@ def _lens_args(lens: Optional[torch.Tensor]):
     return lens.data_ptr(), lens.stride(0)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_current_device = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.current_device
+
+
 def _stream(device) -> int:
     """Handle of torch's current stream on ``device`` (what ``current_stream(device).cuda_stream``
-    returns, without building the Stream object)."""
-    return torch._C._cuda_getCurrentRawStream(device.index)
+    returns, without building the Stream object where this torch has the direct accessor)."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 class _on_device:
@@ -70,7 +76,7 @@ class _on_device:
     __slots__ = ("ctx",)
 
     def __init__(self, device):
-        self.ctx = None if device.index == torch._C._cuda_getDevice() else torch.cuda.device(device)
+        self.ctx = None if device.index == _current_device() else torch.cuda.device(device)
 
     def __enter__(self):
         if self.ctx is not None:
