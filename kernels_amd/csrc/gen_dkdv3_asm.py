@@ -2,7 +2,7 @@
 """Generator of the main-loop assembly of dkdv3_kernel (sa_bwd3.h) -> sa_dkdv3_asm.inc.
 
 The loop body of the dK/dV kernel is a fixed schedule of "slots": each slot issues one
-v_mfma_f32_32x32x16, the LDS read that a slot 7 places later consumes, and a share of the vector
+v_mfma_f32_32x32x16, the LDS read that a slot 15 places later consumes, and a share of the vector
 work of the previous 32-query block.  The compiler's register allocator does not cope with the
 ~400 live registers of that loop (it keeps copying whole accumulators between the two register
 files), so the loop is emitted here with every register chosen by hand, every s_waitcnt counted,
@@ -14,7 +14,7 @@ Register map (the kernel is built for D = 128):
   v[0:31]    lse - score accumulators of the even / odd block   v[32:63]   delta - dP accumulators
   v[64:79]   probabilities, then -dS, of the current block      v[80:95]   free
   v[96:103]  P rounded (two B operands)                         v[104:111] -dS rounded
-  v[112:143] fragment ring, 8 entries of 4 registers
+  v[112:143] fragment ring, entries 0..7 of 4 registers; a[192:223] entries 8..15
   v[144:151] row-fragment addresses, tile of the B side         v[152:159] same, next tile
   v[160:167] transposing-read addresses, tile of the B side     v168, v169 lse/delta addresses (this / next tile)
   v[176:183] row-fragment offsets inside a stage                v[184:191] transposing-read offsets
@@ -35,7 +35,11 @@ Run:  python3 gen_dkdv3_asm.py > sa_dkdv3_asm.inc   (the Makefile does this)
 
 TQ = 64
 RPW = 16
-RING = 8
+import os
+
+# 16 entries let a read be issued up to 15 slots ahead, which is also the most the 4-bit LDS counter of s_waitcnt
+# can keep apart (a transposed fragment is two reads).  8 entries (v[112:143] only) measured 3-5 % slower.
+RING = int(os.environ.get("SA_DKDV3_RING", "16"))
 PF = RING - 1
 
 
@@ -79,7 +83,11 @@ class Gen:
         return self.vr(104 + 4 * half, 4) if w is None else self.vr(104 + 4 * half + w)
 
     def RG(self, r, lo=0, n=4):
-        return self.vr(112 + 4 * r + lo, n)
+        # the second half of the ring lives in accumulation registers: LDS reads can land there and MFMAs can
+        # take their A operand from there
+        if r < 8:
+            return self.vr(112 + 4 * r + lo, n)
+        return self.ar(192 + 4 * (r - 8) + lo, n)
 
     AROW_CUR, AROW_NXT, ATR_CUR, ALD_CUR, ALD_NXT = 144, 152, 160, 168, 169
     AROW_BASE, ATR_BASE, ALD_BASE, QLO, QHI, H4, TMP = 176, 184, 192, 193, 194, 195, 196
@@ -125,7 +133,7 @@ class Gen:
         if j < self.NA:
             g, w = j >> 1, j & 1
             # A side of an odd step is block 0 of the next tile; of an even step block 1 of this tile.
-            # Seen from the step before (which issues slots 0..6), "this tile" of an even step is
+            # Seen from the step before (which issues slots 0..PF-1), "this tile" of an even step is
             # that step's "next tile" until it rotates its address registers, which an odd step does
             # before these reads.
             base = (self.AROW_NXT if par == 1 else self.AROW_CUR) + g
@@ -354,13 +362,13 @@ def generate(D, dt):
         b0 = g.body(k + 1, 0, split_at=split, label=f"e_{D}_{dt}_%=")
         texts = {"B1": b1[0], "B0A": b0[0], "B0B": b0[1]}
         k += 2
-    # prologue: addresses of the first tile, ring entries of the first step's slots 0..6, the first
+    # prologue: addresses of the first tile, ring entries of the first step's slots 0..PF-1, the first
     # block's accumulator starts; everything has returned when it ends
     p = Gen(D, dt)
     pro = [f"v_readfirstlane_b32 s{40 + i}, v{208 + i}" for i in range(len(SCALARS))]
     p.out = pro + p.prologue()
     for j in range(PF):
-        p.fetch(NS + j, j, 1, True)   # same ring positions as any step's slots 0..6 (NS % RING == 0)
+        p.fetch(NS + j, j, 1, True)   # same ring positions as any step's slots 0..PF-1 (NS % RING == 0)
     for rr in range(4):
         p.lds(("lse", 0, rr), f"ds_read_b128 {p.vr(4 * rr, 4)}, v{p.ALD_NXT} offset:{p.row_off(0, 0, rr)}")
     for rr in range(4):
@@ -408,6 +416,7 @@ def generate(D, dt):
 
 def main():
     print("// Generated by gen_dkdv3_asm.py -- do not edit.  Prologue and main loop of dkdv3_kernel.")
+    print("#define SA_DKDV3_RING %d" % RING)
     print("#define SA_DKDV3_NUM_SCALARS %d" % len(SCALARS))
     for i, nm in enumerate(SCALARS):
         print(f"#define SA_DKDV3_SC_{nm.upper()} {i}")
