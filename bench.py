@@ -204,10 +204,10 @@ def cpu_baseline(w, name, budget_s=12.0):
 # inside a timed run, so the figures of the committed summaries under profiles/ are quoted here; a
 # workload or kernel without a committed counter run reports null.
 HBM_BYTES_PER_LAUNCH = {
-    "headline_bf16_T16384_D128": {"fwd": 1.91e+09, "delta": 5.411e+08, "dq": 2.046e+09, "dkdv": 1.712e+09},
-    "bf16_T4096_D64": {"fwd": 2.796e+08, "delta": 1.364e+08, "dq": 3.766e+08, "dkdv": 4.142e+08},
+    "headline_bf16_T16384_D128": {"fwd": 1.909e+09, "delta": 5.411e+08, "dq": 2.051e+09, "dkdv": 1.704e+09},
+    "bf16_T4096_D64": {"fwd": 2.789e+08, "delta": 1.364e+08, "dq": 3.765e+08, "dkdv": 4.141e+08},
     "ragged_fp16_T2048_D128": {"fwd": 1.361e+08, "delta": 1.353e+08, "dq": 1.615e+08, "dkdv": 2.172e+08},
-    "long_bf16_T65536_D128": {"fwd": 1.379e+10, "delta": 1.082e+09, "dq": 1.061e+10, "dkdv": 1.876e+10},
+    "long_bf16_T65536_D128": {"fwd": 1.391e+10, "delta": 1.082e+09, "dq": 1.062e+10, "dkdv": 1.883e+10},
 }
 TRAFFIC_SOURCE = "quoted from the rocprofv3 FETCH_SIZE/WRITE_SIZE summary under profiles/ (not measured in this run)"
 
