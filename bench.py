@@ -342,8 +342,8 @@ def tune_sweep(device, iters=10):
 
 def path_sweep(device, iters=10):
     """Per-kernel times of every (dtype, head dimension) family the library serves, on one shape
-    (B=4, H=16, T=4096, context_size=128, back_contexts=4, lens=None): the 16-bit D in {64, 128}
-    kernels next to the first-generation kernels that serve float32 and D in {16, 32, 256}
+    (B=4, H=16, T=4096, context_size=128, back_contexts=4, lens=None): the 16-bit D in {64, 128, 256}
+    kernels next to the first-generation kernels that serve float32 and D in {16, 32}
     (the reference covers the same range from one tuned kernel, src/streaming_attention/kernel.py:196-203,
     1288-1290).  Rates are executed flop (S and dP are computed by both backward kernels) and
     algorithmic HBM bytes."""

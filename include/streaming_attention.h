@@ -131,9 +131,9 @@ int sa_backward_static(const void* q, const void* k, const void* v,
  *          2: forward key tile (16-bit types)   3: forward key tile (fp32)
  *          4: dQ key tile          5: dK/dV query tile
  *          6: queries (or keys) owned by one workgroup
- *      (1-6 describe the kernels used for float32 and for D in {16, 32, 256})
+ *      (1-6 describe the kernels used for float32 and for D in {16, 32})
  *          7, 8: waves per workgroup of the wide / narrow forward and dQ kernels used for the
- *                16-bit types at D in {64, 128} (each wave owns 32 queries)
+ *                16-bit types at D in {64, 128} (each wave owns 32 queries; D = 256 has the narrow shape only)
  *          9: number of context_size classes of the launch-configuration table (below)
  *         11: number of window classes of that table
  *         10: rows (B*H*T) the static workspace of sa_backward_static holds
@@ -150,7 +150,8 @@ int sa_query(int what);
  *   kernel = 1: dQ        variant 0 = 4 waves, 1 = 8 waves, 2 = software-pipelined kernel (D = 128)
  *   kernel = 2: dK/dV     variant 0 = block-skipping kernel, 1 = software-pipelined kernel (D = 128),
  *                         2 = wave pairs (two waves per SIMD share 32 keys: one forms S and dV, the other dP and dK)
- * sa_launch_choice() returns the variant a call with these sizes runs (-1 for a D outside {64, 128},
+ * sa_launch_choice() returns the variant a call with these sizes runs (always variant 0 at D = 256, whose
+ * kernels exist in one shape; -1 for a D outside {64, 128, 256},
  * a kernel id outside 0..2, context_size < 1 or back_contexts < 0).  Every variant computes the same
  * function. */
 int sa_launch_choice(int D, int context_size, int back_contexts, int kernel);

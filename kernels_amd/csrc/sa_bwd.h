@@ -373,7 +373,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Variants for 16-bit elements with swizzled tiles (D = 64 or 128): tiles arrive by
+// Variants for 16-bit elements with swizzled tiles (D = 64, 128 or 256): tiles arrive by
 // asynchronous global->LDS copies into a ring of NST stages, one barrier per tile.
 // ---------------------------------------------------------------------------------------
 

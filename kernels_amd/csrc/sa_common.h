@@ -425,7 +425,10 @@ template <typename T, int D, int ROWS, int NW, bool ASM_COPIES = false> struct A
   static constexpr int RPI = 1024 / ROW_BYTES;             // rows per instruction
   static constexpr int NI = ROWS / RPI;                     // instructions per tile
   static_assert(ROWS % (RPI * NW) == 0, "tile must split evenly over the waves");
-  static_assert((RPI * NW) % 16 == 0, "the swizzle of a lane must not depend on the instruction");
+  // The swizzle of a lane's row repeats every 16 rows; consecutive instructions of a wave are NW*RPI rows
+  // apart, so a lane needs 16 / (NW*RPI) different offsets when that is less than 16 (wide rows, few waves).
+  static constexpr int NVO = (RPI * NW) % 16 == 0 ? 1 : 16 / (RPI * NW);
+  static_assert((RPI * NW * NVO) % 16 == 0, "the swizzle must repeat after NVO instructions");
   static constexpr int PER_WAVE = NI / NW;                  // instructions per wave per tile
 
   // Buffer addressing: a resource descriptor for the (batch, head) slice whose extent ends with
@@ -439,7 +442,7 @@ template <typename T, int D, int ROWS, int NW, bool ASM_COPIES = false> struct A
   // business either way (wait_loads + barrier).
   u32x4 rsrc;                      // descriptor words for the assembly form
   __amdgpu_buffer_rsrc_t brsrc;    // the same descriptor for the builtin
-  uint32_t voff;      // byte offset of this lane's 16 bytes inside instruction 0 of tile 0
+  uint32_t voff[NVO]; // byte offset of this lane's 16 bytes inside instruction 0 of tile 0 (per swizzle phase)
   uint32_t soff;      // wave-uniform byte offset of the next tile
   uint32_t istep;     // bytes between rows of consecutive instructions of one wave
   uint32_t tstep;     // bytes between consecutive tiles
@@ -455,7 +458,10 @@ template <typename T, int D, int ROWS, int NW, bool ASM_COPIES = false> struct A
     rsrc[2] = (uint32_t)__builtin_amdgcn_readfirstlane((int)bytes);
     rsrc[3] = 0x00020000u;
     brsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gbase), 0, (int)bytes, 0x00020000);
-    voff = ((uint32_t)(wave * RPI + lrow) * rs + (uint32_t)((pch ^ G_::swz(wave * RPI + lrow)) * Elem<T>::VEC)) * ES;
+#pragma unroll
+    for (int j = 0; j < NVO; ++j)
+      voff[j] = ((uint32_t)(wave * RPI + lrow) * rs +
+                 (uint32_t)((pch ^ G_::swz((j * NW + wave) * RPI + lrow)) * Elem<T>::VEC)) * ES;
     soff = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)first_row * rs * ES));
     istep = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(NW * RPI) * rs * ES));
     tstep = (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)ROWS * rs * ES));
@@ -472,10 +478,10 @@ template <typename T, int D, int ROWS, int NW, bool ASM_COPIES = false> struct A
         const uint32_t so = (uint32_t)__builtin_amdgcn_readfirstlane((int)(soff + (uint32_t)i * istep));
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                      :
-                     : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(so)
+                     : "s"(lds_addr), "v"(voff[i % NVO]), "s"(rsrc), "s"(so)
                      : "memory", "m0");
       } else {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(brsrc, (SA_LDS void*)dst, 16, (int)voff,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(brsrc, (SA_LDS void*)dst, 16, (int)voff[i % NVO],
                                                  (int)(soff + (uint32_t)i * istep), 0, 0);
       }
     }

@@ -208,7 +208,7 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
   }
 }
 
-// Forward kernel for 16-bit elements with swizzled tiles (D = 64 or 128).
+// Forward kernel for 16-bit elements with swizzled tiles (D = 64, 128 or 256; at 256 only with 4 waves, one per SIMD, which then has all 512 registers).
 //
 // Same algorithm as fwd_kernel, different resource balance: each wave owns QB blocks of 32
 // queries, so every K / V fragment fetched from LDS feeds QB MFMAs (the transposing V reads

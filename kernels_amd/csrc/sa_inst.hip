@@ -92,7 +92,12 @@ template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
     // windows of less than 1024 keys (the table's first two window classes) run the short-window form
-    const bool wide = launch_choice(D, p.C, p.R).fwd == FWD_WIDE;
+    // head dimension 256 exists in the 4-wave shape only: a wave then has all 512 registers of its SIMD lane
+    const bool wide = D <= 128 && launch_choice(D, p.C, p.R).fwd == FWD_WIDE;
+    if constexpr (D > 128) {
+      if (window_class(p.C, p.R) <= 1) return fwd2_launch<D, C::NARROW_NW, true>(p, st);
+      return fwd2_launch<D, C::NARROW_NW, false>(p, st);
+    }
     if (window_class(p.C, p.R) <= 1)
       return wide ? fwd2_launch<D, C::WIDE_NW, true>(p, st) : fwd2_launch<D, C::NARROW_NW, true>(p, st);
     return wide ? fwd2_launch<D, C::WIDE_NW, false>(p, st) : fwd2_launch<D, C::NARROW_NW, false>(p, st);
@@ -169,6 +174,7 @@ template <int D> static int dq_d(BwdParams p, hipStream_t st) {
     if constexpr (D == 128) {
       if (launch_choice(D, p.C, p.R).dq == DQ_PIPELINED) return dq3_launch<D>(p, st);
     }
+    if constexpr (D > 128) return dq2_launch<D, C::NARROW_NW>(p, st);
     return launch_choice(D, p.C, p.R).dq == DQ_WIDE ? dq2_launch<D, C::WIDE_NW>(p, st) : dq2_launch<D, C::NARROW_NW>(p, st);
   } else {
     constexpr int TQ = C::NW * 32;
@@ -212,7 +218,7 @@ template <int D> static int dkdv3_launch(BwdParams p, hipStream_t st) {
 // wave pairs: 8 waves (two per SIMD) own 128 keys
 template <int D> static int dkdv_split_launch(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
-  if constexpr (C::fwd2(D)) {
+  if constexpr (C::fwd2(D) && D <= 128) {
     constexpr int TKB = 128, TQ = 64, NST = 3, NW = 8;
     // tile stages followed by the pairs' exchange slots; the epilogue's row patches reuse the stages
     constexpr size_t stages = (size_t)NST * (2 * TQ * D * sizeof(ElemT) + 2 * TQ * sizeof(float));

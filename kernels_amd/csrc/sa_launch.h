@@ -40,7 +40,7 @@ template <typename T, int DGROUP> int launch_dkdv(const BwdParams& p, int D, hip
 #define SA_FWD2_NST 2
 #endif
 // ---- launch-configuration table -------------------------------------------------------------------
-// The 16-bit kernels for head dimensions 64 and 128 exist in several shapes; which one runs is read
+// The 16-bit kernels for head dimensions 64 and 128 exist in several shapes (256 in one); which one runs is read
 // from a table indexed by head dimension, chunk-size class and window-size class.  The entries are
 // the fastest variant measured on an MI355X at B=4, H=16, T=16384 (`bench.py --tune-sweep`, turned into
 // sa_tune_table.inc by gen_tune_table.py); float16 and bfloat16 measured alike and share the entries.
@@ -68,6 +68,8 @@ constexpr int window_class(int chunk, int back) {
 // Variants pinned through sa_tune_override() for measurements; -1 = use the table.
 extern int g_tune_override[3];
 inline LaunchChoice launch_choice(int D, int chunk, int back) {
+  // head dimension 256 has one shape per kernel: anything wider or deeper does not fit registers or LDS
+  if (D == 256) return LaunchChoice{FWD_NARROW, DQ_NARROW, DKDV_BLOCKSKIP};
   LaunchChoice c = (D == 128 ? TUNE_D128 : TUNE_D64)[chunk_class(chunk)][window_class(chunk, back)];
   if (g_tune_override[0] >= 0 && g_tune_override[0] < FWD_VARIANTS) c.fwd = g_tune_override[0];
   if (g_tune_override[1] >= 0 && g_tune_override[1] < DQ_VARIANTS) c.dq = g_tune_override[1];
@@ -79,7 +81,7 @@ inline LaunchChoice launch_choice(int D, int chunk, int back) {
 
 template <typename T> struct Cfg {
   static constexpr int NW = 4;                                   // waves per workgroup
-  // 16-bit, D in {64, 128}: forward kernel with QB query blocks per wave and NST LDS stages
+  // 16-bit, D in {64, 128, 256}: forward kernel with QB query blocks per wave and NST LDS stages
   // The forward and dQ kernels come in two widths: 8 waves (256 queries) share each key tile among
   // more waves, which pays once the workgroup's queries lie in one chunk; with smaller chunks the
   // union of the waves' windows grows and 4 waves (128 queries) waste less of every tile.
@@ -95,7 +97,7 @@ template <typename T> struct Cfg {
 #ifdef SA_FWD2_DISABLE
   static constexpr bool fwd2(int) { return false; }
 #else
-  static constexpr bool fwd2(int D) { return sizeof(T) == 2 && (D == 64 || D == 128); }
+  static constexpr bool fwd2(int D) { return sizeof(T) == 2 && (D == 64 || D == 128 || D == 256); }
 #endif
 #ifdef SA_FWD_TK16
   static constexpr int FWD_TK = sizeof(T) == 4 ? 32 : SA_FWD_TK16;

@@ -32,11 +32,11 @@ def _dtype_id(dtype: torch.dtype) -> int:
 def _kernel_layout(t: torch.Tensor) -> torch.Tensor:
     """Return ``t`` itself when the kernels can read it in place (unit stride along the head
     dimension, every other stride and the base address a multiple of 16 bytes, a non-zero stride
-    along T), otherwise a contiguous copy.  The 16-bit kernels for head dimensions 64 and 128
+    along T), otherwise a contiguous copy.  The 16-bit kernels for head dimensions 64 and up
     address the rows of one (batch, head) slice with 32-bit byte offsets (a contiguous tensor is
     within that range up to tens of millions of positions); the other kernels have no such limit."""
     es = t.element_size()
-    offsets32 = es == 2 and t.shape[-1] in (64, 128)
+    offsets32 = es == 2 and t.shape[-1] >= 64
     if t.is_contiguous() and t.data_ptr() % _VEC_BYTES == 0 and t.shape[-1] * es % _VEC_BYTES == 0 \
             and (not offsets32 or (t.shape[-2] + 1024) * t.shape[-1] * es < 2**32):
         return t          # the common case, without looking at every stride

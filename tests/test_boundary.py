@@ -54,6 +54,7 @@ def test_query_and_error_strings(lib):
                 assert lib.sa_launch_choice(D, C, R, 0) in (0, 1)
                 assert lib.sa_launch_choice(D, C, R, 1) in ((0, 1, 2) if D == 128 else (0, 1))
                 assert lib.sa_launch_choice(D, C, R, 2) in ((0, 1, 2) if D == 128 else (0, 2))
+    assert [lib.sa_launch_choice(256, 256, 8, k) for k in range(3)] == [0, 0, 0]
     assert lib.sa_launch_choice(32, 64, 1, 0) == -1 and lib.sa_launch_choice(128, 0, 1, 0) == -1
     assert lib.sa_launch_choice(128, 64, 1, 3) == -1 and lib.sa_launch_choice(128, 64, -1, 0) == -1
     assert lib.sa_tune_override(0, 2) == -3 and lib.sa_tune_override(3, 0) == -3

@@ -120,21 +120,23 @@ def test_all_head_dims(D, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("D", [128, 256])
 @pytest.mark.parametrize("T,C,R", [(257, 64, 2), (513, 128, 1), (300, 256, 8), (1000, 96, 3), (640, 32, 20)])
-def test_tile_edges_16bit(T, C, R, dtype):
+def test_tile_edges_16bit(T, C, R, D, dtype):
     """Lengths and chunk sizes that straddle the kernels' 32/64/128/256-wide tiles."""
-    B, H, D = 2, 2, 128
+    B, H = 2, 2
     q, k, v, d_o = make_inputs(B, H, T, D, seed=22, dtype=dtype)
     lens = torch.tensor([T, max(1, T - 65)], dtype=torch.int32)
     check_against_dense(q, k, v, d_o, lens, C, R, dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [64, 128, 256])
 @pytest.mark.parametrize("C,R", [(16, 2), (20, 300), (48, 30), (100, 3), (200, 0), (200, 1), (300, 4), (600, 0), (1100, 1)])
 def test_every_table_class_16bit(C, R, D, dtype):
     """One context_size per class of the launch-configuration table, windows in all four window
-    classes (48 ... 6020 keys), run with the variants the table picks."""
+    classes (48 ... 6020 keys), run with the variants the table picks (head dimension 256 has one shape
+    per kernel, in the short- and long-window forms)."""
     B, H, T = 2, 2, 1500
     q, k, v, d_o = make_inputs(B, H, T, D, seed=31, dtype=dtype)
     lens = torch.tensor([T, T - 333], dtype=torch.int32)
