@@ -5,7 +5,7 @@ TEST INFRASTRUCTURE ONLY -- the product path never imports this file.
 Three independent formulations of the same operator, so that a mistake in one
 (a dropped term, a wrong sign, a transposed operand) is caught by the others:
 
-* ``dense_f64``       explicit numpy float64 masked softmax and the closed-form
+* ``dense_f64``       explicit float64 masked softmax (CPU tensors) and the closed-form
                       gradients (follows src/streaming_attention/kernel.py:1540-1551
                       for the mask, :239 for the ``lens`` clamp, :408 for the
                       base-2 log-sum-exp, :1017-1022 and :1119-1128 for dS/dQ/dK/dV).
@@ -75,11 +75,6 @@ def unmasked_pairs(T: int, context_size: int, back_contexts: int, L) -> int:
     return total
 
 
-def _round_like(x, dtype):
-    """float64 array -> rounded to ``dtype`` (torch) -> float64."""
-    return torch.from_numpy(np.ascontiguousarray(x)).to(dtype).double().numpy()
-
-
 def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=None, round_dtype=None):
     """Explicit float64 evaluation.  Returns dict with O, LSE (log2 units, 0 at padded
     rows) and, when ``d_out`` is given, dQ, dK, dV (all numpy float64).
@@ -89,41 +84,44 @@ def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=N
     the second matrix products (the reference does the same: kernel.py:370, 1020, 1121, 1127), the
     softmax denominator sums the rounded probabilities, and O is rounded before delta is formed.
     The difference between the two evaluations is the error that rounding alone causes."""
-    qn, kn, vn = (t.detach().cpu().double().numpy() for t in (q, k, v))
+    qn, kn, vn = (t.detach().cpu().double() for t in (q, k, v))
     B, H, T, D = qn.shape
     s = float(D) ** -0.5 if sm_scale is None else float(sm_scale)
     L = clamp_lens(lens, B, T)
-    mask = allowed_mask(T, context_size, back_contexts, L)[:, None]   # [B,1,T,T]
-    S = np.einsum("bhid,bhjd->bhij", qn, kn) * s
-    S = np.where(mask, S, -np.inf)
-    row_valid = mask.any(-1, keepdims=True)                           # [B,1,T,1]
-    m = np.where(row_valid, S.max(-1, keepdims=True, initial=-np.inf), 0.0)
-    E = np.where(mask, np.exp(S - m), 0.0)
-    if round_dtype is not None:
-        E = _round_like(E, round_dtype)
-    l = E.sum(-1, keepdims=True)
-    P = np.where(row_valid, E / np.where(l == 0, 1.0, l), 0.0)
-    O = np.einsum("bhij,bhjd->bhid", P, vn)
-    lse = np.where(row_valid, (m + np.log(np.where(l == 0, 1.0, l))) * LOG2E, 0.0)[..., 0]
-    lse = np.broadcast_to(lse, (B, H, T)).copy()
-    out = {"O": O, "LSE": lse, "P": P}
+    # float64 torch tensors on the CPU: the same arithmetic as numpy, on all host threads
+    mask = torch.from_numpy(allowed_mask(T, context_size, back_contexts, L))[:, None]   # [B,1,T,T]
+    neg_inf = float("-inf")
+
+    def rounded(x):
+        return x if round_dtype is None else x.to(round_dtype).double()
+
+    S = torch.matmul(qn, kn.transpose(-1, -2)) * s
+    S = torch.where(mask, S, neg_inf)
+    row_valid = mask.any(-1, keepdim=True)                            # [B,1,T,1]
+    m = torch.where(row_valid, S.amax(-1, keepdim=True), 0.0)
+    E = rounded(torch.where(mask, torch.exp(S - m), 0.0))
+    l = E.sum(-1, keepdim=True)
+    l_safe = torch.where(l == 0, 1.0, l)
+    P = torch.where(row_valid, E / l_safe, 0.0)
+    O = torch.matmul(P, vn)
+    lse = torch.where(row_valid, (m + torch.log(l_safe)) * LOG2E, 0.0)[..., 0]
+    lse = lse.broadcast_to((B, H, T)).contiguous()
+    out = {"O": O.numpy(), "LSE": lse.numpy(), "P": P.numpy()}
     if d_out is not None:
-        g = d_out.detach().cpu().double().numpy()
-        g = np.broadcast_to(g, O.shape)
+        g = d_out.detach().cpu().double().broadcast_to(O.shape)
         if round_dtype is None:
             Pb, Ob = P, O
         else:
             # backward: P is rebuilt from the saved log-sum-exp and rounded for dV; O was stored rounded
-            Pb = np.where(mask, np.exp(S - lse[..., None] / LOG2E), 0.0) * row_valid
-            Ob = _round_like(O, round_dtype)
-        delta = (Ob * g).sum(-1, keepdims=True)
-        dP = np.einsum("bhid,bhjd->bhij", g, vn)
+            Pb = torch.where(mask, torch.exp(S - lse[..., None] / LOG2E), 0.0) * row_valid
+            Ob = rounded(O)
+        delta = (Ob * g).sum(-1, keepdim=True)
+        dP = torch.matmul(g, vn.transpose(-1, -2))
         dS = Pb * (dP - delta)
-        if round_dtype is not None:
-            Pb, dS = _round_like(Pb, round_dtype), _round_like(dS, round_dtype)
-        out["dV"] = np.einsum("bhij,bhid->bhjd", Pb, g)
-        out["dQ"] = s * np.einsum("bhij,bhjd->bhid", dS, kn)
-        out["dK"] = s * np.einsum("bhij,bhid->bhjd", dS, qn)
+        Pb, dS = rounded(Pb), rounded(dS)
+        out["dV"] = torch.matmul(Pb.transpose(-1, -2), g).numpy()
+        out["dQ"] = (s * torch.matmul(dS, kn)).numpy()
+        out["dK"] = (s * torch.matmul(dS.transpose(-1, -2), qn)).numpy()
     return out
 
 
