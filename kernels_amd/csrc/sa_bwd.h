@@ -192,8 +192,16 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(const BwdParams p) {
   }
 }
 
-template <typename T, int D, int NW, int TQ>
+// PASS selects what one launch produces: 0 both gradients, 1 dV only, 2 dK only.  Two float32 accumulators of 32 x 256
+// and the resident K and V rows are 512 registers per lane before any operand, so float32 at head dimension 256 runs
+// as two launches: the dV pass needs neither V nor dP, the dK pass has one accumulator and stages the next tile in two
+// halves (Q while the first products run, dO during the rest), so that only one tile's worth of staging registers is
+// live at a time (with both halves live, the compiler's spill code for the first tile lost a value).
+template <typename T, int D, int NW, int TQ, int PASS = 0>
 __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
+  constexpr bool WITH_DV = PASS != 2, WITH_DK = PASS != 1;
+  constexpr bool HALVES = PASS == 2;   // stage Q and dO one after the other
+  static_assert(!HALVES || TQ == 32, "the two staging halves bracket a single 32-query block");
   using E = Elem<T>;
   using G = TileGeom<T, D>;
   using Frag = typename E::Frag;
@@ -224,8 +232,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   T* dv_base = reinterpret_cast<T*>(p.dv) + (int64_t)bh * T_ * D;
   const int k_end = k0 + TKB < T_ ? k0 + TKB : T_;
   if (k0 >= L) {
-    zero_rows<T, D, NT>(dk_base, k0, k_end, tid);
-    zero_rows<T, D, NT>(dv_base, k0, k_end, tid);
+    if constexpr (WITH_DK) zero_rows<T, D, NT>(dk_base, k0, k_end, tid);
+    if constexpr (WITH_DV) zero_rows<T, D, NT>(dv_base, k0, k_end, tid);
     return;
   }
 
@@ -247,7 +255,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   const float sl2e = fabsf(p.scale_log2e);
   const bool neg = p.scale_log2e < 0.0f;
 
-  Frag kf[NF], vf[NF];
+  Frag kf[NF], vf[WITH_DK ? NF : 1];
   {
     const int kr = krow < L ? krow : L - 1;
     const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.k_sb + (int64_t)hd * p.k_sh +
@@ -258,7 +266,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
     for (int g = 0; g < NF; ++g) {
       kf[g] = *reinterpret_cast<const Frag*>(kp + (g * 2 + h) * E::VEC);
       if (neg) kf[g] = negate<T>(kf[g]);
-      vf[g] = *reinterpret_cast<const Frag*>(vp + (g * 2 + h) * E::VEC);
+      if constexpr (WITH_DK) vf[g] = *reinterpret_cast<const Frag*>(vp + (g * 2 + h) * E::VEC);
     }
   }
 
@@ -267,11 +275,14 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   const float* lse_base = p.lse + (int64_t)bh * T_;
   const float* delta_base = p.delta + (int64_t)bh * T_;
 
-  f32x16 dk[DB], dv[DB];
+  f32x16 dk[WITH_DK ? DB : 1], dv[WITH_DV ? DB : 1];
 #pragma unroll
   for (int m = 0; m < DB; ++m)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
+    for (int i = 0; i < 16; ++i) {
+      if constexpr (WITH_DK) dk[m][i] = 0.0f;
+      if constexpr (WITH_DV) dv[m][i] = 0.0f;
+    }
 
   Stager<T, D, TQ, NT> sq, sg;
   float r_lse = 0.0f, r_delta = 0.0f;   // thread tid < TQ stages row tid of the tile
@@ -286,7 +297,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   auto stage_ptr = [&](int s) { return smem_raw + s * STAGE_BYTES; };
   auto store_stage = [&](int s) {
     T* qd = reinterpret_cast<T*>(stage_ptr(s));
-    sq.store(qd, tid);
+    if constexpr (!HALVES) sq.store(qd, tid);
     sg.store(qd + TILE, tid);
     if (tid < TQ) {
       float* f = reinterpret_cast<float*>(stage_ptr(s) + 2 * TILE * sizeof(T));
@@ -297,6 +308,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   static_assert(TQ <= NW * 64, "one thread per staged row");
 
   sq.load(qbase, p.q_st, qt0 * TQ, L - 1, tid);
+  if constexpr (HALVES) sq.store(reinterpret_cast<T*>(stage_ptr(0)), tid);
   sg.load(gbase, p.do_st, qt0 * TQ, L - 1, tid);
   load_rows(qt0 * TQ);
   store_stage(0);
@@ -312,7 +324,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
     const bool more = t + 1 < qt1;
     if (more) {
       sq.load(qbase, p.q_st, (t + 1) * TQ, L - 1, tid);
-      sg.load(gbase, p.do_st, (t + 1) * TQ, L - 1, tid);
+      if constexpr (!HALVES) sg.load(gbase, p.do_st, (t + 1) * TQ, L - 1, tid);
       load_rows((t + 1) * TQ);
     }
     const int qs = t * TQ;
@@ -328,7 +340,16 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
         f32x16 (&s1)[1] = reinterpret_cast<f32x16(&)[1]>(s);
         f32x16 (&dp1)[1] = reinterpret_cast<f32x16(&)[1]>(dp);
         mma_rows<T, D>(s1, Qt, qb * 32, kf, lane);
-        mma_rows<T, D>(dp1, Gt, qb * 32, vf, lane);
+        if constexpr (WITH_DK) mma_rows<T, D>(dp1, Gt, qb * 32, vf, lane);
+      }
+      if constexpr (HALVES) {
+        // the other stage has had no reader since the last barrier: Q goes there now, dO takes over the registers
+        sched_fence();   // the loads below must not be moved up into the products
+        if (more) {
+          sq.store(reinterpret_cast<T*>(stage_ptr(cur ^ 1)), tid);
+          sg.load(gbase, p.do_st, (t + 1) * TQ, L - 1, tid);
+        }
+        sched_fence();
       }
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
@@ -352,8 +373,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
         }
       }
       // dV^T[d][key] += dO^T P,  dK^T[d][key] += Q^T dS
-      mma_tr<T, D>(dv, Gt, qb, s, lane);
-      mma_tr<T, D>(dk, Qt, qb, dp, lane);
+      if constexpr (WITH_DV) mma_tr<T, D>(dv, Gt, qb, s, lane);
+      if constexpr (WITH_DK) mma_tr<T, D>(dk, Qt, qb, dp, lane);
     }
 
     if (more) store_stage(cur ^ 1);
@@ -365,10 +386,13 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
 #pragma unroll
       for (int m = 0; m < DB; ++m)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dk[m][i] = 0.0f, dv[m][i] = 0.0f;
+        for (int i = 0; i < 16; ++i) {
+          if constexpr (WITH_DK) dk[m][i] = 0.0f;
+          if constexpr (WITH_DV) dv[m][i] = 0.0f;
+        }
     }
-    store_acc_T<T, D, DB>(dk_base + (int64_t)krow * D, dk, p.scale, h);
-    store_acc_T<T, D, DB>(dv_base + (int64_t)krow * D, dv, 1.0f, h);
+    if constexpr (WITH_DK) store_acc_T<T, D, DB>(dk_base + (int64_t)krow * D, dk, p.scale, h);
+    if constexpr (WITH_DV) store_acc_T<T, D, DB>(dv_base + (int64_t)krow * D, dv, 1.0f, h);
   }
 }
 

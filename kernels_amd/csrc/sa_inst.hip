@@ -264,14 +264,27 @@ template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
     constexpr int TKB = C::NW * 32;
     constexpr size_t lds =
         (size_t)2 * (2 * C::DKDV_TQ * TileGeom<ElemT, D>::PITCH * sizeof(ElemT) + 2 * C::DKDV_TQ * sizeof(float));
-    auto kern = dkdv_kernel<ElemT, D, C::NW, C::DKDV_TQ>;
-    static PrepareState once;
-    if (int rc = prepare(kern, lds, once)) return rc;
     p.n_tiles = (int)ceil_div(p.T, TKB);
     const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
     if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
-    return (int)hipGetLastError();
+    if constexpr (sizeof(ElemT) == 4 && D == 256) {
+      // both accumulators and both resident rows do not fit a lane's registers: one launch per gradient
+      auto kern_dv = dkdv_kernel<ElemT, D, C::NW, C::DKDV_TQ, 1>;
+      auto kern_dk = dkdv_kernel<ElemT, D, C::NW, C::DKDV_TQ, 2>;
+      static PrepareState once_dv, once_dk;
+      if (int rc = prepare(kern_dv, lds, once_dv)) return rc;
+      if (int rc = prepare(kern_dk, lds, once_dk)) return rc;
+      hipLaunchKernelGGL(kern_dv, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
+      if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+      hipLaunchKernelGGL(kern_dk, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
+      return (int)hipGetLastError();
+    } else {
+      auto kern = dkdv_kernel<ElemT, D, C::NW, C::DKDV_TQ>;
+      static PrepareState once;
+      if (int rc = prepare(kern, lds, once)) return rc;
+      hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(C::NW * 64), lds, st, p);
+      return (int)hipGetLastError();
+    }
   }
 }
 template <> int launch_dkdv<ElemT, SA_DGROUP>(const BwdParams& p, int D, hipStream_t st) {
