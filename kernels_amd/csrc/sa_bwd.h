@@ -194,9 +194,10 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(const BwdParams p) {
 
 // PASS selects what one launch produces: 0 both gradients, 1 dV only, 2 dK only.  Two float32 accumulators of 32 x 256
 // and the resident K and V rows are 512 registers per lane before any operand, so float32 at head dimension 256 runs
-// as two launches: the dV pass needs neither V nor dP, the dK pass has one accumulator and stages the next tile in two
-// halves (Q while the first products run, dO during the rest), so that only one tile's worth of staging registers is
-// live at a time (with both halves live, the compiler's spill code for the first tile lost a value).
+// as two launches: the dV pass needs neither V nor dP and fits without spills; the dK pass has one accumulator and
+// stages the next tile in two steps (Q while the first products run, dO during the rest).  It still spills some values
+// around the products; the form that staged both tensors at once was miscompiled (the spill code of the first tile
+// dropped a register copy), which the head-dimension parity tests catch.
 template <typename T, int D, int NW, int TQ, int PASS = 0>
 __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   constexpr bool WITH_DV = PASS != 2, WITH_DK = PASS != 1;

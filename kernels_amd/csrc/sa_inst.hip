@@ -93,14 +93,15 @@ template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
   if constexpr (C::fwd2(D)) {
     // windows of less than 1024 keys (the table's first two window classes) run the short-window form
     // head dimension 256 exists in the 4-wave shape only: a wave then has all 512 registers of its SIMD lane
-    const bool wide = D <= 128 && launch_choice(D, p.C, p.R).fwd == FWD_WIDE;
     if constexpr (D > 128) {
       if (window_class(p.C, p.R) <= 1) return fwd2_launch<D, C::NARROW_NW, true>(p, st);
       return fwd2_launch<D, C::NARROW_NW, false>(p, st);
+    } else {
+      const bool wide = launch_choice(D, p.C, p.R).fwd == FWD_WIDE;
+      if (window_class(p.C, p.R) <= 1)
+        return wide ? fwd2_launch<D, C::WIDE_NW, true>(p, st) : fwd2_launch<D, C::NARROW_NW, true>(p, st);
+      return wide ? fwd2_launch<D, C::WIDE_NW, false>(p, st) : fwd2_launch<D, C::NARROW_NW, false>(p, st);
     }
-    if (window_class(p.C, p.R) <= 1)
-      return wide ? fwd2_launch<D, C::WIDE_NW, true>(p, st) : fwd2_launch<D, C::NARROW_NW, true>(p, st);
-    return wide ? fwd2_launch<D, C::WIDE_NW, false>(p, st) : fwd2_launch<D, C::NARROW_NW, false>(p, st);
   } else {
     constexpr int TQ = C::NW * 32;
     constexpr size_t lds = (size_t)2 * 2 * C::FWD_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
@@ -175,7 +176,7 @@ template <int D> static int dq_d(BwdParams p, hipStream_t st) {
       if (launch_choice(D, p.C, p.R).dq == DQ_PIPELINED) return dq3_launch<D>(p, st);
     }
     if constexpr (D > 128) return dq2_launch<D, C::NARROW_NW>(p, st);
-    return launch_choice(D, p.C, p.R).dq == DQ_WIDE ? dq2_launch<D, C::WIDE_NW>(p, st) : dq2_launch<D, C::NARROW_NW>(p, st);
+    else return launch_choice(D, p.C, p.R).dq == DQ_WIDE ? dq2_launch<D, C::WIDE_NW>(p, st) : dq2_launch<D, C::NARROW_NW>(p, st);
   } else {
     constexpr int TQ = C::NW * 32;
     constexpr size_t lds = (size_t)2 * 2 * C::DQ_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
