@@ -56,16 +56,11 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
   const int pair = wave & (NP - 1);
   const bool grad_role = wave >= NP;
 
-  int bh, kt;
-  tile_coords(blockIdx.x, gridDim.x, p.n_tiles, bh, kt);
+  int bh, kt, L;
+  key_tile_coords(blockIdx.x, gridDim.x, p.n_tiles, growing_tiles(p.C, p.R, p.T, TKB), TKB, p.H, p.T, p.lens,
+                  p.lens_stride, bh, kt, L);
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
-
-  int L = T_;
-  if (p.lens) {
-    L = p.lens[(int64_t)b * p.lens_stride];
-    L = L < 0 ? 0 : (L > T_ ? T_ : L);
-  }
   const int k0 = kt * TKB;
   T* dk_base = reinterpret_cast<T*>(p.dk) + (int64_t)bh * T_ * D;
   T* dv_base = reinterpret_cast<T*>(p.dv) + (int64_t)bh * T_ * D;

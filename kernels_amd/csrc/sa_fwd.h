@@ -242,7 +242,7 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   int bh, qt;
-  tile_coords(blockIdx.x, gridDim.x, p.n_tiles, bh, qt);
+  tile_coords(blockIdx.x, gridDim.x, p.n_tiles, bh, qt, SHORT ? growing_tiles(p.C, p.R, p.T, NW * QB * 32) : 0);
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
 
