@@ -243,7 +243,7 @@ def test_noncontiguous_inputs(dtype):
         assert_close("dV", vd.grad, ref["dV"], dtype)
 
 
-@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float32, 32)])
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float32, 32), (torch.float16, 256)])
 def test_packed_qkv_projection_is_read_in_place(dtype, D):
     """q, k, v as views of one [B, T, 3, H, D] projection output: no copies on the way in, and the
     gradient arrives in the packed tensor."""
