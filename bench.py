@@ -518,6 +518,9 @@ def main():
         "peaks_used": {"bf16_mfma_tflops": PEAK_BF16_TFLOPS, "f32_mfma_tflops": PEAK_F32_TFLOPS,
                        "hbm_gbs": PEAK_HBM_GBS},
         "kernel_ms": kt,
+        "kernel_ms_note": ("each kernel launched on its own through the C ABI; for this dtype and head dimension the step's "
+                           "backward forms delta inside the dQ kernel and does not launch the delta pass timed here"
+                           if w["dtype"] != "float32" and D >= 64 else "each kernel launched on its own through the C ABI"),
         "kernel_tflops": {n: kernel_flops[n] / (kt[n] * 1e-3) / 1e12 for n in kernel_flops},
         "kernel_gbs": {n: kernel_bytes[n] / (kt[n] * 1e-3) / 1e9 for n in kernel_bytes},
         "roofline": roofline,

@@ -91,8 +91,14 @@ int sa_bwd_dkdv(const void* q, const void* k, const void* v,
                 int context_size, int back_contexts, float sm_scale,
                 int dtype, void* stream);
 
-/* Whole backward = sa_bwd_delta + sa_bwd_dkdv + sa_bwd_dq on one stream; `delta` is a
- * caller-provided [B,H,T] float32 workspace.  Replaces the body of
+/* Whole backward on one stream; `delta` is a caller-provided [B,H,T] float32 workspace that holds
+ * rowsum(O * dO) afterwards.  For float32 and for head dimensions 16 and 32 this is sa_bwd_delta +
+ * sa_bwd_dkdv + sa_bwd_dq.  For float16 / bfloat16 at head dimensions 64, 128 and 256 the dQ kernel
+ * forms the row sums itself from the dO rows it holds anyway (it reads O once more and writes
+ * `delta` for the dK/dV kernel, which runs after it), so the separate pass over O and dO -- the
+ * reference's `_streaming_attn_bwd_precompute` launch, kernel.py:433-514 -- is not launched; the
+ * sums are added in another order than sa_bwd_delta adds them, so the gradients agree with those
+ * of the separate calls to rounding, not bit for bit.  Replaces the body of
  * `attention_backward_adapter` (src/streaming_attention/kernel.py:1363-1442). */
 int sa_backward(const void* q, const void* k, const void* v,
                 const int32_t* lens, int64_t lens_stride,
@@ -105,7 +111,7 @@ int sa_backward(const void* q, const void* k, const void* v,
                 int dtype, void* stream);
 
 /* sa_backward for callers that cannot allocate device memory (code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc): the same three kernels, with the
+ * tight serving loops, harnesses that forbid hipMalloc): the same kernels, with the
  * [B,H,T] float32 row-sum workspace taken from a static device array inside the library instead
  * of a `delta` argument.  It has no counterpart in the reference.
  *   - B*H*T must not exceed SA_STATIC_MAX_ROWS (sa_query(10)); larger problems return

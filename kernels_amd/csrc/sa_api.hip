@@ -129,10 +129,13 @@ static int fill_bwd(BwdParams& p, const void* q, const void* k, const void* v, c
   return SA_OK;
 }
 
-int sa_bwd_dq(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
-              const void* d_o, const float* lse, const float* delta, void* dq, const int64_t* qs,
-              const int64_t* ks, const int64_t* vs, const int64_t* gs, int B, int H, int T, int D,
-              int context_size, int back_contexts, float sm_scale, int dtype, void* stream) {
+// dQ launch.  With o != null the kernel forms delta = rowsum(O * dO) itself and writes it to `delta` for
+// the dK/dV launch that follows (the kernels that can: see delta_inside_dq()).
+static int run_dq(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
+                  const void* d_o, const float* lse, float* delta, void* dq, const int64_t* qs,
+                  const int64_t* ks, const int64_t* vs, const int64_t* gs, int B, int H, int T, int D,
+                  int context_size, int back_contexts, float sm_scale, int dtype, void* stream, const void* o,
+                  const int64_t* os) {
   BwdParams p{};
   if (int rc = fill_bwd(p, q, k, v, lens, lens_stride, d_o, lse, delta, qs, ks, vs, gs, B, H, T, D,
                         context_size, back_contexts, sm_scale, dtype))
@@ -140,9 +143,22 @@ int sa_bwd_dq(const void* q, const void* k, const void* v, const int32_t* lens, 
   if (B == 0 || H == 0 || T == 0) return SA_OK;
   if (!dq || !aligned16(dq)) return dq ? SA_ERR_LAYOUT : SA_ERR_ARG;
   p.dq = dq;
+  if (o) {
+    if (int rc = check_layout(o, os, dtype, T, D)) return rc;
+    p.o = o; p.o_sb = os[0]; p.o_sh = os[1]; p.o_st = os[2];
+    p.delta_out = delta;
+  }
   return by_dtype(dtype, [&](auto tag) {
     using E = decltype(tag);
     return D == 256 ? launch_dq<E, 1>(p, D, (hipStream_t)stream) : launch_dq<E, 0>(p, D, (hipStream_t)stream); });
+}
+
+int sa_bwd_dq(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
+              const void* d_o, const float* lse, const float* delta, void* dq, const int64_t* qs,
+              const int64_t* ks, const int64_t* vs, const int64_t* gs, int B, int H, int T, int D,
+              int context_size, int back_contexts, float sm_scale, int dtype, void* stream) {
+  return run_dq(q, k, v, lens, lens_stride, d_o, lse, const_cast<float*>(delta), dq, qs, ks, vs, gs, B, H, T, D,
+                context_size, back_contexts, sm_scale, dtype, stream, nullptr, nullptr);
 }
 
 int sa_bwd_dkdv(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
@@ -162,17 +178,40 @@ int sa_bwd_dkdv(const void* q, const void* k, const void* v, const int32_t* lens
     return D == 256 ? launch_dkdv<E, 1>(p, D, (hipStream_t)stream) : launch_dkdv<E, 0>(p, D, (hipStream_t)stream); });
 }
 
-int sa_backward(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
-                const void* o, const void* d_o, const float* lse, float* delta, void* dq, void* dk, void* dv,
-                const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os, const int64_t* gs,
-                int B, int H, int T, int D, int context_size, int back_contexts, float sm_scale, int dtype,
-                void* stream) {
+// The dQ kernels for the 16-bit types at head dimensions 64, 128 and 256 hold each query's dO row and form
+// delta = rowsum(O * dO) in their prologue; the separate pass over O and dO is then not launched.
+static bool delta_inside_dq(int D, int dtype) { return dtype != SA_DTYPE_F32 && D >= 64; }
+
+// The launches behind sa_backward and sa_backward_static: delta, dK/dV, dQ -- or dQ (forming delta), dK/dV.
+static int backward_launches(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
+                             const void* o, const void* d_o, const float* lse, float* delta, void* dq, void* dk,
+                             void* dv, const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
+                             const int64_t* gs, int B, int H, int T, int D, int context_size, int back_contexts,
+                             float sm_scale, int dtype, void* stream) {
+  if (int rc = check_common(B, H, T, D, dtype)) return rc;
+  if (delta_inside_dq(D, dtype) && B > 0 && H > 0 && T > 0) {
+    if (!o || !os || !delta) return SA_ERR_ARG;
+    if (int rc = run_dq(q, k, v, lens, lens_stride, d_o, lse, delta, dq, qs, ks, vs, gs, B, H, T, D, context_size,
+                        back_contexts, sm_scale, dtype, stream, o, os))
+      return rc;
+    return sa_bwd_dkdv(q, k, v, lens, lens_stride, d_o, lse, delta, dk, dv, qs, ks, vs, gs, B, H, T, D,
+                       context_size, back_contexts, sm_scale, dtype, stream);
+  }
   if (int rc = sa_bwd_delta(o, d_o, delta, os, gs, B, H, T, D, dtype, stream)) return rc;
   if (int rc = sa_bwd_dkdv(q, k, v, lens, lens_stride, d_o, lse, delta, dk, dv, qs, ks, vs, gs, B, H, T, D,
                            context_size, back_contexts, sm_scale, dtype, stream))
     return rc;
   return sa_bwd_dq(q, k, v, lens, lens_stride, d_o, lse, delta, dq, qs, ks, vs, gs, B, H, T, D, context_size,
                    back_contexts, sm_scale, dtype, stream);
+}
+
+int sa_backward(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
+                const void* o, const void* d_o, const float* lse, float* delta, void* dq, void* dk, void* dv,
+                const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os, const int64_t* gs,
+                int B, int H, int T, int D, int context_size, int back_contexts, float sm_scale, int dtype,
+                void* stream) {
+  return backward_launches(q, k, v, lens, lens_stride, o, d_o, lse, delta, dq, dk, dv, qs, ks, vs, os, gs, B, H, T, D,
+                           context_size, back_contexts, sm_scale, dtype, stream);
 }
 
 int sa_backward_static(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
@@ -200,13 +239,9 @@ int sa_backward_static(const void* q, const void* k, const void* v, const int32_
     delta = base[dev];
   }
   if (!delta) return SA_ERR_ARG;
-  // every row the kernels read is written by the delta pass first: nothing to clear
-  if (int rc = sa_bwd_delta(o, d_o, delta, os, gs, B, H, T, D, dtype, stream)) return rc;
-  if (int rc = sa_bwd_dkdv(q, k, v, lens, lens_stride, d_o, lse, delta, dk, dv, qs, ks, vs, gs, B, H, T, D,
-                           context_size, back_contexts, sm_scale, dtype, stream))
-    return rc;
-  return sa_bwd_dq(q, k, v, lens, lens_stride, d_o, lse, delta, dq, qs, ks, vs, gs, B, H, T, D, context_size,
-                   back_contexts, sm_scale, dtype, stream);
+  // every row the kernels read is written first, by the delta pass or by the dQ kernel: nothing to clear
+  return backward_launches(q, k, v, lens, lens_stride, o, d_o, lse, delta, dq, dk, dv, qs, ks, vs, os, gs, B, H, T, D,
+                           context_size, back_contexts, sm_scale, dtype, stream);
 }
 
 int sa_query(int what) {

@@ -436,6 +436,8 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
   const int q_end = q0 + TQ < T_ ? q0 + TQ : T_;
   if (q0 >= L) {
     zero_rows<T, D, NT>(dq_base, q0, q_end, tid);
+    if (p.delta_out)
+      for (int r = q0 + tid; r < q_end; r += NT) p.delta_out[(int64_t)bh * T_ + r] = 0.0f;
     return;
   }
 
@@ -484,6 +486,18 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
                   (int64_t)qr * p.q_st;
     const T* gp = reinterpret_cast<const T*>(p.d_o) + (int64_t)b * p.do_sb + (int64_t)hd * p.do_sh +
                   (int64_t)qr * p.do_st;
+    // delta = rowsum(O * dO) is formed here when the caller has not run the delta kernel: this lane holds half
+    // of its query's dO row, so the forward output is fetched in the same pattern, in flight together with the
+    // other rows, and the two halves are added across lanes
+    Frag of[NF];
+    if (p.delta_out) {
+      const T* op = reinterpret_cast<const T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)hd * p.o_sh + (int64_t)qr * p.o_st;
+#pragma unroll
+      for (int g = 0; g < NF; ++g) of[g] = *reinterpret_cast<const Frag*>(op + (g * 2 + h) * E::VEC);
+    } else {
+#pragma unroll
+      for (int g = 0; g < NF; ++g) of[g] = Frag{};
+    }
 #pragma unroll
     for (int g = 0; g < NF; ++g) {
       qf[g] = *reinterpret_cast<const Frag*>(qp + (g * 2 + h) * E::VEC);
@@ -493,7 +507,15 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
       gf[g] = negate<T>(*reinterpret_cast<const Frag*>(gp + (g * 2 + h) * E::VEC));
     }
     lse_q = qrow < L ? p.lse[(int64_t)bh * T_ + qr] : INFINITY;   // rows past L: P = exp2(-inf) = 0
-    delta_q = p.delta[(int64_t)bh * T_ + qr];
+    if (p.delta_out) {
+      float osum = 0.0f;
+#pragma unroll
+      for (int g = 0; g < NF; ++g) osum = dot_frag(of[g], gf[g], osum);
+      delta_q = -half_sum(osum);
+      if (h == 0 && qrow < T_) p.delta_out[(int64_t)bh * T_ + qrow] = qrow < L ? delta_q : 0.0f;
+    } else {
+      delta_q = p.delta[(int64_t)bh * T_ + qr];
+    }
   }
   f32x16 dinit;
 #pragma unroll

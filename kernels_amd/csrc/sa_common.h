@@ -151,6 +151,21 @@ SA_DEV float sum_frag(bf16x8 f, float acc) {
     acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{f[2 * j], f[2 * j + 1]}, one, acc, false);
   return acc;
 }
+// acc + the dot product of two fragments, two elements per instruction, products and sums in float32
+SA_DEV float dot_frag(bf16x8 a, bf16x8 b, float acc) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    acc = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{a[2 * j], a[2 * j + 1]}, bf16x2{b[2 * j], b[2 * j + 1]}, acc, false);
+  return acc;
+}
+SA_DEV float dot_frag(f16x8 a, f16x8 b, float acc) {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    acc = __builtin_amdgcn_fdot2(f16x2{a[2 * j], a[2 * j + 1]}, f16x2{b[2 * j], b[2 * j + 1]}, acc, false);
+  return acc;
+}
 SA_DEV float sum_frag(f16x8 f, float acc) {
   typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
   const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
@@ -714,6 +729,11 @@ struct BwdParams {
   int B, H, T, C, R;
   float scale, scale_log2e;
   int n_tiles;
+  // Set only for a dQ kernel that forms the row sums itself (delta_out != null): the forward output, its
+  // element strides, and where the sums go for the dK/dV kernel that runs after it.  `delta` is then unused.
+  const void* o;
+  int64_t o_sb, o_sh, o_st;
+  float* delta_out;
 };
 
 struct DeltaParams {

@@ -178,6 +178,7 @@ template <int D> static int dq_d(BwdParams p, hipStream_t st) {
     if constexpr (D > 128) return dq2_launch<D, C::NARROW_NW>(p, st);
     else return launch_choice(D, p.C, p.R).dq == DQ_WIDE ? dq2_launch<D, C::WIDE_NW>(p, st) : dq2_launch<D, C::NARROW_NW>(p, st);
   } else {
+    if (p.delta_out) return SA_ERR_ARG;
     constexpr int TQ = C::NW * 32;
     constexpr size_t lds = (size_t)2 * 2 * C::DQ_TK * TileGeom<ElemT, D>::PITCH * sizeof(ElemT);
     auto kern = dq_kernel<ElemT, D, C::NW, C::DQ_TK>;

@@ -458,13 +458,20 @@ def test_c_abi_direct_calls():
         assert_close(name, got, ref[name], dtype)
     want_delta = (ref["O"] * d_o.double().cpu().numpy()).sum(-1)
     assert_close("delta", delta, want_delta, dtype)
-    # sa_backward = the three launches behind one entry point
+    # sa_backward = the launches behind one entry point.  For 16-bit inputs at this head dimension the dQ
+    # kernel forms delta itself (another summation order than the delta kernel's), so the results agree
+    # with the separate launches to rounding, not bit for bit; the workspace holds the same row sums.
     dq2, dk2, dv2 = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    delta.fill_(float("nan"))
     assert lib.sa_backward(q.data_ptr(), k.data_ptr(), v.data_ptr(), lens.data_ptr(), 1, o.data_ptr(), d_o.data_ptr(),
                            lse.data_ptr(), delta.data_ptr(), dq2.data_ptr(), dk2.data_ptr(), dv2.data_ptr(),
                            s4(q), s4(k), s4(v), s4(o), s4(d_o), B, H, T, D, C, R, sc, 2, st) == 0
     torch.cuda.synchronize()
-    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+    for name, got in (("dQ", dq2), ("dK", dk2), ("dV", dv2)):
+        assert_close(name, got, ref[name], dtype)
+    for got, sep in ((dq2, dq), (dk2, dk), (dv2, dv)):
+        assert (got.float() - sep.float()).abs().max().item() <= 2e-2
+    assert_close("delta", delta, want_delta, dtype)
     # a layout the kernels cannot read in place is refused, not mis-read
     assert lib.sa_forward(q.data_ptr() + 2, k.data_ptr(), v.data_ptr(), None, 0, o.data_ptr(), None,
                           s4(q), s4(k), s4(v), B, H, T, D, C, R, sc, 2, st) == -4
