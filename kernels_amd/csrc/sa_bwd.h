@@ -489,15 +489,14 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
     // delta = rowsum(O * dO) is formed here when the caller has not run the delta kernel: this lane holds half
     // of its query's dO row, so the forward output is fetched in the same pattern, in flight together with the
     // other rows, and the two halves are added across lanes
+    // (no branch around the loads: a value defined on one side only is copied where the sides join, and the copy
+    // waits for the load; without a row of O to read, the dO row is read twice)
     Frag of[NF];
-    if (p.delta_out) {
-      const T* op = reinterpret_cast<const T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)hd * p.o_sh + (int64_t)qr * p.o_st;
+    const T* op = p.delta_out ? reinterpret_cast<const T*>(p.o) + (int64_t)b * p.o_sb + (int64_t)hd * p.o_sh +
+                                    (int64_t)qr * p.o_st
+                              : gp;
 #pragma unroll
-      for (int g = 0; g < NF; ++g) of[g] = *reinterpret_cast<const Frag*>(op + (g * 2 + h) * E::VEC);
-    } else {
-#pragma unroll
-      for (int g = 0; g < NF; ++g) of[g] = Frag{};
-    }
+    for (int g = 0; g < NF; ++g) of[g] = *reinterpret_cast<const Frag*>(op + (g * 2 + h) * E::VEC);
 #pragma unroll
     for (int g = 0; g < NF; ++g) {
       qf[g] = *reinterpret_cast<const Frag*>(qp + (g * 2 + h) * E::VEC);
@@ -507,11 +506,11 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
       gf[g] = negate<T>(*reinterpret_cast<const Frag*>(gp + (g * 2 + h) * E::VEC));
     }
     lse_q = qrow < L ? p.lse[(int64_t)bh * T_ + qr] : INFINITY;   // rows past L: P = exp2(-inf) = 0
-    if (p.delta_out) {
-      float osum = 0.0f;
+    float osum = 0.0f;
 #pragma unroll
-      for (int g = 0; g < NF; ++g) osum = dot_frag(of[g], gf[g], osum);
-      delta_q = -half_sum(osum);
+    for (int g = 0; g < NF; ++g) osum = dot_frag(of[g], gf[g], osum);
+    delta_q = -half_sum(osum);
+    if (p.delta_out) {
       if (h == 0 && qrow < T_) p.delta_out[(int64_t)bh * T_ + qrow] = qrow < L ? delta_q : 0.0f;
     } else {
       delta_q = p.delta[(int64_t)bh * T_ + qr];
