@@ -204,10 +204,10 @@ def cpu_baseline(w, name, budget_s=12.0):
 # inside a timed run, so the figures of the committed summaries under profiles/ are quoted here; a
 # workload or kernel without a committed counter run reports null.
 HBM_BYTES_PER_LAUNCH = {
-    "headline_bf16_T16384_D128": {"fwd": 1.911e+09, "delta": 5.411e+08, "dq": 1.808e+09, "dkdv": 1.749e+09},
-    "bf16_T4096_D64": {"fwd": 3.069e+08, "delta": 1.364e+08, "dq": 4.198e+08, "dkdv": 4.38e+08},
-    "ragged_fp16_T2048_D128": {"fwd": 1.413e+08, "delta": 1.353e+08, "dq": 1.639e+08, "dkdv": 2.199e+08},
-    "long_bf16_T65536_D128": {"fwd": 1.39e+10, "delta": 1.082e+09, "dq": 8.398e+09, "dkdv": 5.753e+09},
+    "headline_bf16_T16384_D128": {"fwd": 1.921e+09, "delta": 5.411e+08, "dq": 1.894e+09, "dkdv": 1.761e+09},
+    "bf16_T4096_D64": {"fwd": 3.105e+08, "delta": 1.364e+08, "dq": 4.84e+08, "dkdv": 4.4e+08},
+    "ragged_fp16_T2048_D128": {"fwd": 1.414e+08, "delta": 1.353e+08, "dq": 1.775e+08, "dkdv": 2.193e+08},
+    "long_bf16_T65536_D128": {"fwd": 1.377e+10, "delta": 1.082e+09, "dq": 8.774e+09, "dkdv": 5.758e+09},
 }
 TRAFFIC_SOURCE = "quoted from the rocprofv3 FETCH_SIZE/WRITE_SIZE summary under profiles/ (not measured in this run)"
 
