@@ -583,6 +583,9 @@ template <typename T, int D, int NW, int TQ, int NST>
 // H=16, T=4096).  At 128 the same step (290 -> 256 registers) spills inside the products and is 40 % slower.
 __global__ __launch_bounds__(NW * 64, (D == 64 ? 3 : 1)) void dkdv2_kernel(const BwdParams p) {
   using E = Elem<T>;
+  // fragments fetched ahead of the MFMAs, per group: two at head dimension 64, where the smaller groups let the kernel
+  // fit the 168 registers of three waves per SIMD with one reloaded value instead of six (another 5 % faster)
+  constexpr int PG = D == 64 ? 2 : 4;
   using G = TileGeom<T, D>;
   using Frag = typename E::Frag;
   static_assert(G::SWZ && (NST == 2 || NST == 3), "swizzled 16-bit tiles, 2 or 3 stages");
@@ -720,7 +723,7 @@ __global__ __launch_bounds__(NW * 64, (D == 64 ? 3 : 1)) void dkdv2_kernel(const
         for (int e = 0; e < 4; ++e) s[0][4 * g4 + e] = l4[e], dp[0][4 * g4 + e] = d4[e];
       }
       // S[q][key] = Q K^T and dP[q][key] = dO V^T
-      mma_rows_pair<T, D>(s[0], dp[0], Qt, Gt, qb * 32, kf, vf, lane);
+      mma_rows_pair<T, D, NF, PG>(s[0], dp[0], Qt, Gt, qb * 32, kf, vf, lane);
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
 #pragma unroll
@@ -741,7 +744,7 @@ __global__ __launch_bounds__(NW * 64, (D == 64 ? 3 : 1)) void dkdv2_kernel(const
         }
       }
       // dV^T[d][key] += dO^T P and -dK^T[d][key] += Q^T (-dS)
-      mma_tr_pair<T, D>(dv, dk, Gt, Qt, qb, s[0], dp[0], lane);
+      mma_tr_pair<T, D, DB, PG>(dv, dk, Gt, Qt, qb, s[0], dp[0], lane);
     }
   }
 

@@ -337,7 +337,7 @@ template <typename T> SA_DEV void pack_c(typename Elem<T>::Frag (&b)[2], const f
 // Two products that share the pipeline: acc0 += A0 * B0 and acc1 += A1 * B1, where A0 and A1
 // are the same 32 rows of two row-major LDS tiles (scores from Q and K, dP from dO and V).
 // One fragment stream means one exposed LDS latency instead of two.
-template <typename T, int D, int NF>
+template <typename T, int D, int NF, int GRP = 4>
 SA_DEV void mma_rows_pair(f32x16& acc0, f32x16& acc1, const T* tile0, const T* tile1, int row0,
                           const typename Elem<T>::Frag (&b0)[NF], const typename Elem<T>::Frag (&b1)[NF],
                           int lane) {
@@ -346,7 +346,7 @@ SA_DEV void mma_rows_pair(f32x16& acc0, f32x16& acc1, const T* tile0, const T* t
   static_assert(NF == G_::NF, "one register fragment per 2*VEC slice of the head dimension");
   constexpr int PITCH = G_::PITCH, VEC = Elem<T>::VEC;
   const int c = lane & 31, h = lane >> 5;
-  constexpr int N = 2 * NF, G = N < 4 ? N : 4;
+  constexpr int N = 2 * NF, G = N < GRP ? N : GRP;
   const int off = (row0 + c) * PITCH;
   const int sw = G_::swz(c);
   pipeline<N, G>(
@@ -362,7 +362,7 @@ SA_DEV void mma_rows_pair(f32x16& acc0, f32x16& acc1, const T* tile0, const T* t
 
 // Likewise for the transposed products: acc0[m] += X0^T * P0 and acc1[m] += X1^T * P1 over the
 // same 32-row block of two tiles (dV from dO and P, dK from Q and dS).  16-bit types only.
-template <typename T, int D, int NM>
+template <typename T, int D, int NM, int GRP = 4>
 SA_DEV void mma_tr_pair(f32x16 (&acc0)[NM], f32x16 (&acc1)[NM], const T* X0, const T* X1, int rb,
                         const f32x16& P0, const f32x16& P1, int lane) {
   using E = Elem<T>;
@@ -376,7 +376,7 @@ SA_DEV void mma_tr_pair(f32x16 (&acc0)[NM], f32x16 (&acc1)[NM], const T* X0, con
   Frag b0[2], b1[2];
   pack_c<T>(b0, P0);
   pack_c<T>(b1, P1);
-  constexpr int N = 4 * NM, G = N < 4 ? N : 4;
+  constexpr int N = 4 * NM, G = N < GRP ? N : GRP;
   pipeline<N, G>(
       [&](int it) {
         const int k2 = it % (2 * NM), half = k2 / NM, m = k2 % NM;
