@@ -204,10 +204,10 @@ def cpu_baseline(w, name, budget_s=12.0):
 # inside a timed run, so the figures of the committed summaries under profiles/ are quoted here; a
 # workload or kernel without a committed counter run reports null.
 HBM_BYTES_PER_LAUNCH = {
-    "headline_bf16_T16384_D128": {"fwd": 1.918e+09, "delta": 5.411e+08, "dq": 1.934e+09, "dkdv": 1.755e+09},
-    "bf16_T4096_D64": {"fwd": 3.136e+08, "delta": 1.364e+08, "dq": 4.846e+08, "dkdv": 6.023e+08},
-    "ragged_fp16_T2048_D128": {"fwd": 1.415e+08, "delta": 1.353e+08, "dq": 1.774e+08, "dkdv": 2.195e+08},
-    "long_bf16_T65536_D128": {"fwd": 1.371e+10, "delta": 1.082e+09, "dq": 8.6e+09, "dkdv": 5.775e+09},
+    "headline_bf16_T16384_D128": {"fwd": 1.914e+09, "delta": 5.411e+08, "dq": 1.927e+09, "dkdv": 1.747e+09},
+    "bf16_T4096_D64": {"fwd": 3.072e+08, "delta": 1.364e+08, "dq": 4.847e+08, "dkdv": 5.352e+08},
+    "ragged_fp16_T2048_D128": {"fwd": 1.415e+08, "delta": 1.353e+08, "dq": 1.775e+08, "dkdv": 2.195e+08},
+    "long_bf16_T65536_D128": {"fwd": 1.378e+10, "delta": 1.082e+09, "dq": 8.672e+09, "dkdv": 5.757e+09},
 }
 TRAFFIC_SOURCE = "quoted from the rocprofv3 FETCH_SIZE/WRITE_SIZE summary under profiles/ (not measured in this run)"
 
