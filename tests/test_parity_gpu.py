@@ -287,6 +287,36 @@ def test_backward_op_accepts_foreign_gradient_and_missing_lse():
     assert_close("dV", dv, ref["dV"], dtype)
 
 
+@pytest.mark.parametrize("D,T,C,R", [(64, 200, 16, 2), (128, 700, 256, 8)])
+def test_backward_op_reads_a_strided_forward_output(D, T, C, R):
+    """The backward op with the forward output stored [B,T,H,D] (read in place through its strides): for
+    16-bit inputs the dQ kernels form delta = rowsum(O * dO) from it themselves -- the narrow dQ kernel at
+    D=64, the software-pipelined one at D=128 with a 2304-key window."""
+    from streaming_attention import _lib
+    from streaming_attention.ops import _kernel_layout
+
+    dev = torch.device("cuda:0")
+    B, H = 2, 2
+    dtype = torch.bfloat16
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=33, dtype=dtype)
+    lens = torch.tensor([T, T - 59], dtype=torch.int32)
+    if D == 128:
+        assert _lib.load().sa_launch_choice(D, C, R, 1) == 2
+    qd, kd, vd = (t.to(dev) for t in (q, k, v))
+    fwd = torch.ops.alexdremov_streaming_attention.forward
+    bwd = torch.ops.alexdremov_streaming_attention.backward
+    o, lse = fwd(qd, kd, vd, lens.to(dev), C, R, D ** -0.5, False, True, False, "ieee")
+    o_bthd = o.transpose(1, 2).contiguous().transpose(1, 2)
+    assert not o_bthd.is_contiguous() and _kernel_layout(o_bthd) is o_bthd
+    dq, dk, dv = bwd(qd, kd, vd, lens.to(dev), o_bthd, lse, d_o.to(dev), C, R, D ** -0.5, False, False, "ieee")
+    ref = sa_oracle.dense_f64(q, k, v, lens, C, R, d_out=d_o)
+    assert_close("dQ", dq, ref["dQ"], dtype)
+    assert_close("dK", dk, ref["dK"], dtype)
+    assert_close("dV", dv, ref["dV"], dtype)
+    dq2, dk2, dv2 = bwd(qd, kd, vd, lens.to(dev), o, lse, d_o.to(dev), C, R, D ** -0.5, False, False, "ieee")
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+
+
 def check_rounding_aware(q, k, v, d_o, lens, C, R, dtype, sm_scale=None, record=None):
     """16-bit results against the float64 oracle with the bar widened by what rounding P and dS to
     the input type costs in a float64 evaluation of the same formulas (no input is changed to fit)."""
