@@ -154,6 +154,42 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
   for (int i = 0; i < 16; ++i) dp[0][i] = 0.0f;
 
   char* const xbuf = smem_raw + XBUF_OFF + pair * 2 * XSLOT + lane * 16;
+
+  // Byte offsets of this lane's fragments inside a tile, block 0: row-major fragment g of row c, and the two
+  // transposing reads (rows r_lo and r_lo + 8 of the first 16) of column block m.  The swizzle of a row depends
+  // on its low four bits only, so every other block of a tile is a compile-time distance away and an LDS read
+  // costs one address addition; left to itself the compiler rebuilds the swizzled address for every read.
+  uint32_t row_off[NF], tr_off[2][DB];
+  {
+    const int g16 = lane >> 4, j = lane & 15;
+    const int r_lo = 4 * (g16 >> 1) + (j >> 2), col = (g16 & 1) * 16 + 4 * (j & 3);
+#pragma unroll
+    for (int g = 0; g < NF; ++g) row_off[g] = (uint32_t)G::off(c, (g * 2 + h) * E::VEC) * (uint32_t)sizeof(T);
+#pragma unroll
+    for (int m = 0; m < DB; ++m) {
+      tr_off[0][m] = (uint32_t)G::off(r_lo, m * 32 + col) * (uint32_t)sizeof(T);
+      tr_off[1][m] = (uint32_t)G::off(r_lo + 8, m * 32 + col) * (uint32_t)sizeof(T);
+    }
+  }
+  constexpr int BLOCK_BYTES = 32 * G::PITCH * (int)sizeof(T);   // 32 rows of a tile
+  // accS += rows [32 qb, 32 qb + 32) of the tile at byte offset `tile` of the LDS allocation, times rf
+  auto rows_product = [&](f32x16& accS, int tile, int qb) {
+    const char* base = smem_raw + tile + qb * BLOCK_BYTES;
+    pipeline<NF, GRP>([&](int g) { return *reinterpret_cast<const Frag*>(base + row_off[g]); },
+                      [&](int g, const Frag& a) { mma(accS, a, rf[g]); });
+  };
+  // accD[m] += (rows [32 qb, 32 qb + 32) of that tile)^T times the packed block b
+  auto tr_product = [&](f32x16 (&accD)[DB], int tile, int qb, const Frag (&b)[2]) {
+    const char* base = smem_raw + tile + qb * BLOCK_BYTES;
+    pipeline<2 * DB, GRP>(
+        [&](int it) {
+          const char* p = base + (it / DB) * (BLOCK_BYTES / 2);
+          s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p + tr_off[0][it % DB]));
+          s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((SA_LDS s16x4*)(p + tr_off[1][it % DB]));
+          return __builtin_bit_cast(Frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        },
+        [&](int it, const Frag& a) { mma(accD[it % DB], a, b[it / DB]); });
+  };
   wait_all_loads();
 
   // lse (WHICH = 0) or delta (WHICH = 1) of the 16 rows of block qb this lane holds in a C fragment
@@ -187,15 +223,14 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
     auto step = [&](int t, int qb) {
       const int g = 2 * t + qb;
       if (!blk_live(g)) return;
-      const T* Qt = reinterpret_cast<const T*>(smem_raw + st_cur);
-      const T* Gt = Qt + TILE;
       const float* ld_t = reinterpret_cast<const float*>(smem_raw + st_cur + 2 * TILE * sizeof(T));
       f32x16 s[1];
       rows16(ld_t, qb, 0, s[0]);
-      mma_rows<T, D, 1, NF, GRP>(s, Qt, qb * 32, rf, lane);        // lse - S[q][key]
+      rows_product(s[0], st_cur, qb);                              // lse - S[q][key]
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[0][i] = fast_exp2(-s[0][i]);
       if (!blk_interior(g)) {
+        asm volatile("");   // a real branch: as straight-line selects the mask would cost every block 3 instructions per score
         const uint32_t rm = row_mask(qlo - g * 32, qhi - g * 32, h);
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[0][i] = keep_or_zero(s[0][i], keep_bits(rm, i));
@@ -205,7 +240,7 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
       char* slot = xbuf + (g & 1) * XSLOT;
       *reinterpret_cast<Frag*>(slot) = pf[0][0];
       *reinterpret_cast<Frag*>(slot + 1024) = pf[0][1];
-      mma_tr_n<T, D, 1, DB, GRP>(acc, Gt, qb, pf, lane);          // dV^T[d][key] += dO^T P
+      tr_product(acc[0], st_cur + TILE * (int)sizeof(T), qb, pf[0]);   // dV^T[d][key] += dO^T P
     };
     for (int t = qt0; t < qt1; ++t) {
       wait_tile(t);
@@ -225,7 +260,6 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
       const int g = 2 * t + qb;
       const bool cur = t < qt1 && blk_live(g);
       const bool prev = g > 2 * qt0 && blk_live(g - 1);
-      const T* Gt = reinterpret_cast<const T*>(smem_raw + st_cur) + TILE;
       const float* ld_t = reinterpret_cast<const float*>(smem_raw + st_cur + 2 * TILE * sizeof(T));
       // dS of the previous block first: its delta - dP leaves the registers that the next product fills
       Frag df[1][2];
@@ -243,11 +277,10 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
       }
       if (cur) {
         rows16(ld_t, qb, 1, dp[0]);
-        mma_rows<T, D, 1, NF, GRP>(dp, Gt, qb * 32, rf, lane);     // delta - dP[q][key]
+        rows_product(dp[0], st_cur + TILE * (int)sizeof(T), qb);   // delta - dP[q][key]
       }
       if (prev) {
-        const T* Qp = reinterpret_cast<const T*>(smem_raw + (qb ? st_cur : st_prev));
-        mma_tr_n<T, D, 1, DB, GRP>(acc, Qp, qb ? 0 : 1, df, lane);   // -dK^T[d][key] += Q^T (-dS)
+        tr_product(acc[0], qb ? st_cur : st_prev, qb ? 0 : 1, df[0]);   // -dK^T[d][key] += Q^T (-dS)
       }
     };
     for (int t = qt0; t < qt1; ++t) {
