@@ -105,8 +105,8 @@ def make_inputs(name, device, zeros=False):
                 lens_list=lens_list, B=B, H=H, T=T, D=D, C=C, R=R, dtype=dtype_name)
 
 
-def time_kernels(w, iters):
-    """Average duration of each kernel launched on its own through the C ABI, in ms."""
+def time_kernels(w, iters, only=None):
+    """Average duration of each kernel (or of those named in `only`) launched on its own through the C ABI, in ms."""
     import torch
     from streaming_attention import _lib
 
@@ -142,6 +142,8 @@ def time_kernels(w, iters):
 
     out = {}
     for name, fn in (("fwd", fwd), ("delta", dlt), ("dq", dqf), ("dkdv", dkv)):
+        if only is not None and name not in only:
+            continue
         _lib.check(fn(), name)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -152,6 +154,10 @@ def time_kernels(w, iters):
         e1.synchronize()
         out[name] = e0.elapsed_time(e1) / iters
     return out
+
+
+def time_kernels_only(w, iters, only):
+    return time_kernels(w, iters, only)
 
 
 def cpu_baseline(w, name, budget_s=12.0):
@@ -297,7 +303,7 @@ def tune_sweep(device, iters=10):
 
     lib = _lib.load()
     B, H, T = 4, 16, 16384
-    names = {"fwd": ["narrow", "wide"], "dq": ["narrow", "wide", "pipelined"], "dkdv": ["blockskip", "pipelined", "split"]}
+    names = {"fwd": ["narrow", "pipelined"], "dq": ["narrow", "pipelined"], "dkdv": ["blockskip", "pipelined", "split"]}
     rows = []
     try:
         for dtype_name in ("bfloat16", "float16"):

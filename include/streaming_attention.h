@@ -23,7 +23,16 @@
  *     the caller need not clear them first.  Input positions t >= lens[b] are never
  *     read, so they may hold anything.
  *   - Return value: 0 on success, > 0 a hipError_t from the launch, < 0 one of SA_ERR_*.
- *   - Re-entrant; no global mutable state apart from one-time kernel attribute set-up.
+ *   - Re-entrant.  The library's mutable state is the per-device, per-kernel attribute set-up
+ *     (hipFuncSetAttribute on the first call of each kernel shape on each device, guarded by a
+ *     mutex) and the variants pinned through sa_tune_override() (atomics; a measurement and test
+ *     hook that no product caller needs).  Because of the former, the first call of each kernel
+ *     shape on a device must be made outside a HIP graph capture.
+ *   - The 16-bit dK/dV kernels at D >= 64 multiply K by -sm_scale*log2(e) and round the product to the
+ *     element type before the score MFMA (what the reference does for prescale_qk=True,
+ *     src/streaming_attention/kernel.py:1065-1066), whatever `prescale_qk` the caller of the Python
+ *     operator passed: their probabilities differ from the forward's by about |score| * 2^-9 (bf16) /
+ *     2^-12 (fp16) relative, inside the 16-bit accuracy bar.  Forward and dQ scale in float32.
  */
 #ifndef STREAMING_ATTENTION_H
 #define STREAMING_ATTENTION_H
@@ -138,8 +147,10 @@ int sa_backward_static(const void* q, const void* k, const void* v,
  *          4: dQ key tile          5: dK/dV query tile
  *          6: queries (or keys) owned by one workgroup
  *      (1-6 describe the kernels used for float32 and for D in {16, 32})
- *          7, 8: waves per workgroup of the wide / narrow forward and dQ kernels used for the
- *                16-bit types at D in {64, 128} (each wave owns 32 queries; D = 256 has the narrow shape only)
+ *          7: 1 when the hand-scheduled (software-pipelined) kernels are part of this build, 0 when it was
+ *             compiled with SA_NO_ASM_KERNELS and serves every call with the compiler-scheduled kernels
+ *          8: waves per workgroup of the compiler-scheduled forward and dQ kernels used for the
+ *             16-bit types at D in {64, 128, 256} (each wave owns 32 queries)
  *          9: number of context_size classes of the launch-configuration table (below)
  *         11: number of window classes of that table
  *         10: rows (B*H*T) the static workspace of sa_backward_static holds
@@ -152,8 +163,9 @@ int sa_query(int what);
  * outcome of an offline sweep on MI355X, indexed by head dimension, context_size class
  * (< 32, < 64, < 128, < 256, < 512, < 1024, >= 1024) and window class
  * (context_size * (back_contexts + 1) < 256, < 1024, < 4096, >= 4096).
- *   kernel = 0: forward   variant 0 = 4 waves (128 queries) per workgroup, 1 = 8 waves (256 queries)
- *   kernel = 1: dQ        variant 0 = 4 waves, 1 = 8 waves, 2 = software-pipelined kernel (D = 128)
+ *   kernel = 0: forward   variant 0 = 4 waves (128 queries) per workgroup, 1 = software-pipelined kernel
+ *                         (D = 128: 4 waves of 64 queries, one wave per SIMD)
+ *   kernel = 1: dQ        variant 0 = 4 waves (128 queries), 1 = software-pipelined kernel (D = 128)
  *   kernel = 2: dK/dV     variant 0 = block-skipping kernel, 1 = software-pipelined kernel (D = 128),
  *                         2 = wave pairs (two waves per SIMD share 32 keys: one forms S and dV, the other dP and dK)
  * sa_launch_choice() returns the variant a call with these sizes runs (always variant 0 at D = 256, whose
@@ -166,7 +178,9 @@ int sa_launch_choice(int D, int context_size, int back_contexts, int kernel);
  * variant = -1.  Meant for measurements (it is how the table was produced) and for tests that
  * exercise every variant; the counterpart of the reference's `autotune` switch
  * (src/streaming_attention/kernel.py:1154-1193).  A pinned software-pipelined variant applies to D = 128 only.
- * Not synchronised with launches on other threads.  Returns 0 or SA_ERR_ARG. */
+ * A measurement and test hook, not part of the operator: the pinned variants are the library's only
+ * mutable state besides the per-device kernel attributes.  They are atomics, so a launch on another
+ * thread sees either the old or the new variant, but which one is not ordered.  Returns 0 or SA_ERR_ARG. */
 int sa_tune_override(int kernel, int variant);
 
 /* Human-readable text for a return code of the functions above (static storage). */

@@ -12,7 +12,7 @@ using namespace sa;
 static __device__ __align__(256) float sa_static_delta[SA_STATIC_MAX_ROWS];
 
 namespace sa {
-int g_tune_override[3] = {-1, -1, -1};
+std::atomic<int> g_tune_override[3] = {{-1}, {-1}, {-1}};
 }
 
 namespace {
@@ -180,7 +180,7 @@ int sa_bwd_dkdv(const void* q, const void* k, const void* v, const int32_t* lens
 
 // The dQ kernels for the 16-bit types at head dimensions 64, 128 and 256 hold each query's dO row and form
 // delta = rowsum(O * dO) in their prologue; the separate pass over O and dO is then not launched.
-static bool delta_inside_dq(int D, int dtype) { return dtype != SA_DTYPE_F32 && D >= 64; }
+static bool delta_inside_dq(int D, int dtype) { return dtype != SA_DTYPE_F32 && Cfg<__bf16>::fwd2(D); }
 
 // The launches behind sa_backward and sa_backward_static: delta, dK/dV, dQ -- or dQ (forming delta), dK/dV.
 static int backward_launches(const void* q, const void* k, const void* v, const int32_t* lens, int64_t lens_stride,
@@ -189,8 +189,17 @@ static int backward_launches(const void* q, const void* k, const void* v, const 
                              const int64_t* gs, int B, int H, int T, int D, int context_size, int back_contexts,
                              float sm_scale, int dtype, void* stream) {
   if (int rc = check_common(B, H, T, D, dtype)) return rc;
+  if (B > 0 && H > 0 && T > 0) {
+    // every output is checked before the first launch: nothing is enqueued for a call that is going to fail
+    if (!dq || !dk || !dv || !delta) return SA_ERR_ARG;
+    if (!aligned16(dq) || !aligned16(dk) || !aligned16(dv)) return SA_ERR_LAYOUT;
+    if (int rc = check_layout(o, os, dtype, T, D)) return rc;
+    BwdParams probe{};
+    if (int rc = fill_bwd(probe, q, k, v, lens, lens_stride, d_o, lse, delta, qs, ks, vs, gs, B, H, T, D,
+                          context_size, back_contexts, sm_scale, dtype))
+      return rc;
+  }
   if (delta_inside_dq(D, dtype) && B > 0 && H > 0 && T > 0) {
-    if (!o || !os || !delta) return SA_ERR_ARG;
     if (int rc = run_dq(q, k, v, lens, lens_stride, d_o, lse, delta, dq, qs, ks, vs, gs, B, H, T, D, context_size,
                         back_contexts, sm_scale, dtype, stream, o, os))
       return rc;
@@ -253,7 +262,7 @@ int sa_query(int what) {
     case 4: return Cfg<__bf16>::DQ_TK;
     case 5: return Cfg<__bf16>::DKDV_TQ;
     case 6: return Cfg<__bf16>::NW * 32;
-    case 7: return Cfg<__bf16>::WIDE_NW;
+    case 7: return kAsmKernels ? 1 : 0;
     case 8: return Cfg<__bf16>::NARROW_NW;
     case 9: return TUNE_CHUNK_CLASSES;
     case 10: return SA_STATIC_MAX_ROWS;
@@ -272,7 +281,7 @@ int sa_tune_override(int kernel, int variant) {
   if (kernel < 0 || kernel > 2) return SA_ERR_ARG;
   const int limit = kernel == 0 ? FWD_VARIANTS : kernel == 1 ? DQ_VARIANTS : DKDV_VARIANTS;
   if (variant < -1 || variant >= limit) return SA_ERR_ARG;
-  g_tune_override[kernel] = variant;
+  g_tune_override[kernel].store(variant, std::memory_order_relaxed);
   return SA_OK;
 }
 

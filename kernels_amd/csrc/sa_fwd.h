@@ -411,8 +411,15 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
 #pragma unroll
           for (int i = 0; i < 16; ++i) pr[i] = fast_exp2(__builtin_fmaf(s[qb][kb][i], sl2e, -m_use));
           pack_c<T>(pb[qb][kb], pr);
+#ifdef SA_FWD2_DOT_SUMS
           rs[0] = sum_frag(pb[qb][kb][0], rs[0]);
           rs[1] = sum_frag(pb[qb][kb][1], rs[1]);
+#else
+          // plain float32 additions in two chains: the two-element dot products that could add up the rounded
+          // values at half the instruction count stall against the MFMAs in flight
+#pragma unroll
+          for (int i = 0; i < 16; i += 2) rs[0] += pr[i], rs[1] += pr[i + 1];
+#endif
         }
       };
       // A wave none of whose lanes has a maximum yet (its first visible tile) goes straight to the

@@ -6,10 +6,15 @@
 #include "sa_launch.h"
 #if SA_KIND == 0
 #include "sa_fwd.h"
+#ifndef SA_NO_ASM_KERNELS
+#include "sa_fwd3.h"
+#endif
 #else
 #include "sa_bwd.h"
+#ifndef SA_NO_ASM_KERNELS
 #include "sa_bwd3.h"
 #include "sa_bwd4.h"
+#endif
 #include "sa_bwd_split.h"
 #endif
 
@@ -88,19 +93,45 @@ template <int D, int NW, bool SHORT> static int fwd2_launch(FwdParams p, hipStre
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), lds, st, p);
   return (int)hipGetLastError();
 }
+// hand-scheduled loop, one wave per SIMD, 64 queries per wave (head dimension 128)
+template <int D> static int fwd3_launch(FwdParams p, hipStream_t st) {
+#ifdef SA_NO_ASM_KERNELS
+  (void)p; (void)st;
+  return SA_ERR_HEAD_DIM;
+#else
+  using C = Cfg<ElemT>;
+  if constexpr (C::fwd2(D) && D == 128) {
+    constexpr int NW = 4, TQ = NW * 64, NST = 4;
+    constexpr size_t stages = (size_t)NST * 2 * 64 * D * sizeof(ElemT);
+    constexpr size_t patches = (size_t)NW * RowPatch<ElemT, D>::ELEMS * sizeof(ElemT);
+    constexpr size_t lds = stages > patches ? stages : patches;
+    auto kern = fwd3_kernel<ElemT, D, NST>;
+    static PrepareState once;
+    if (int rc = prepare(kern, lds, once)) return rc;
+    p.n_tiles = (int)ceil_div(p.T, TQ);
+    const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), lds, st, p);
+    return (int)hipGetLastError();
+  } else {
+    return SA_ERR_HEAD_DIM;
+  }
+#endif
+}
 template <int D> static int fwd_d(FwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
+    if constexpr (D == 128) {
+      if (launch_choice(D, p.C, p.R).fwd == FWD_PIPELINED) return fwd3_launch<D>(p, st);
+    }
     // windows of less than 1024 keys (the table's first two window classes) run the short-window form
     // head dimension 256 exists in the 4-wave shape only: a wave then has all 512 registers of its SIMD lane
     if constexpr (D > 128) {
       if (window_class(p.C, p.R) <= 1) return fwd2_launch<D, C::NARROW_NW, true>(p, st);
       return fwd2_launch<D, C::NARROW_NW, false>(p, st);
     } else {
-      const bool wide = launch_choice(D, p.C, p.R).fwd == FWD_WIDE;
-      if (window_class(p.C, p.R) <= 1)
-        return wide ? fwd2_launch<D, C::WIDE_NW, true>(p, st) : fwd2_launch<D, C::NARROW_NW, true>(p, st);
-      return wide ? fwd2_launch<D, C::WIDE_NW, false>(p, st) : fwd2_launch<D, C::NARROW_NW, false>(p, st);
+      if (window_class(p.C, p.R) <= 1) return fwd2_launch<D, C::NARROW_NW, true>(p, st);
+      return fwd2_launch<D, C::NARROW_NW, false>(p, st);
     }
   } else {
     constexpr int TQ = C::NW * 32;
@@ -151,6 +182,10 @@ template <int D, int NW> static int dq2_launch(BwdParams p, hipStream_t st) {
 }
 // hand-scheduled loop, one wave per SIMD, 64 queries per wave (head dimension 128)
 template <int D> static int dq3_launch(BwdParams p, hipStream_t st) {
+#ifdef SA_NO_ASM_KERNELS
+  (void)p; (void)st;
+  return SA_ERR_HEAD_DIM;
+#else
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D) && D == 128) {
     constexpr int NW = 4, TQ = NW * 64, NST = 4;
@@ -168,6 +203,7 @@ template <int D> static int dq3_launch(BwdParams p, hipStream_t st) {
   } else {
     return SA_ERR_HEAD_DIM;
   }
+#endif
 }
 template <int D> static int dq_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
@@ -175,8 +211,7 @@ template <int D> static int dq_d(BwdParams p, hipStream_t st) {
     if constexpr (D == 128) {
       if (launch_choice(D, p.C, p.R).dq == DQ_PIPELINED) return dq3_launch<D>(p, st);
     }
-    if constexpr (D > 128) return dq2_launch<D, C::NARROW_NW>(p, st);
-    else return launch_choice(D, p.C, p.R).dq == DQ_WIDE ? dq2_launch<D, C::WIDE_NW>(p, st) : dq2_launch<D, C::NARROW_NW>(p, st);
+    return dq2_launch<D, C::NARROW_NW>(p, st);
   } else {
     if (p.delta_out) return SA_ERR_ARG;
     constexpr int TQ = C::NW * 32;
@@ -198,6 +233,10 @@ template <> int launch_dq<ElemT, SA_DGROUP>(const BwdParams& p, int D, hipStream
 }
 #else
 template <int D> static int dkdv3_launch(BwdParams p, hipStream_t st) {
+#ifdef SA_NO_ASM_KERNELS
+  (void)p; (void)st;
+  return SA_ERR_HEAD_DIM;
+#else
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D) && D == 128) {
     constexpr int TKB = 128, TQ = 64;
@@ -216,6 +255,7 @@ template <int D> static int dkdv3_launch(BwdParams p, hipStream_t st) {
   } else {
     return SA_ERR_HEAD_DIM;
   }
+#endif
 }
 // wave pairs: 8 waves (two per SIMD) own 128 keys
 template <int D> static int dkdv_split_launch(BwdParams p, hipStream_t st) {

@@ -1,6 +1,7 @@
 // Host-side launch entry points, one explicit instantiation per element type.
 // Each returns 0, a positive hipError_t, or a negative SA_ERR_* code.
 #pragma once
+#include <atomic>
 #include "../../include/streaming_attention.h"
 #include "sa_common.h"
 
@@ -45,11 +46,11 @@ template <typename T, int DGROUP> int launch_dkdv(const BwdParams& p, int D, hip
 // the fastest variant measured on an MI355X at B=4, H=16, T=16384 (`bench.py --tune-sweep`, turned into
 // sa_tune_table.inc by gen_tune_table.py); float16 and bfloat16 measured alike and share the entries.
 enum FwdVariant : int { FWD_NARROW = 0,     // 4 waves (128 queries) per workgroup, two workgroups per CU
-                        FWD_WIDE = 1,       // 8 waves (256 queries) share every key tile
+                        FWD_PIPELINED = 1,  // hand-scheduled loop, 4 waves of 64 queries (head dimension 128 only)
                         FWD_VARIANTS = 2 };
-enum DqVariant : int { DQ_NARROW = 0, DQ_WIDE = 1,
-                       DQ_PIPELINED = 2,   // hand-scheduled loop, 4 waves of 64 queries (head dimension 128 only)
-                       DQ_VARIANTS = 3 };
+enum DqVariant : int { DQ_NARROW = 0,      // 4 waves (128 queries) per workgroup
+                       DQ_PIPELINED = 1,   // hand-scheduled loop, 4 waves of 64 queries (head dimension 128 only)
+                       DQ_VARIANTS = 2 };
 enum DkdvVariant : int { DKDV_BLOCKSKIP = 0,   // every wave skips the query tiles outside its own 32 keys' windows
                          DKDV_PIPELINED = 1,   // hand-scheduled loop, head dimension 128 only
                          DKDV_SPLIT = 2,       // wave pairs share 32 keys: one wave forms S and dV, the other dP and dK
@@ -65,27 +66,41 @@ constexpr int window_class(int chunk, int back) {
   return w < 256 ? 0 : w < 1024 ? 1 : w < 4096 ? 2 : 3;
 }
 #include "sa_tune_table.inc"
-// Variants pinned through sa_tune_override() for measurements; -1 = use the table.
-extern int g_tune_override[3];
+// Variants pinned through sa_tune_override() for measurements and tests; -1 = use the table.  The only
+// mutable state of the library besides the per-device kernel attributes: atomics, so that a launch on
+// one thread reads a whole value while another thread pins or releases a variant.
+extern std::atomic<int> g_tune_override[3];
+// The hand-scheduled kernels are single assembly statements over fixed registers.  A build with
+// -DSA_NO_ASM_KERNELS leaves them out (for a compiler that cannot satisfy their register constraints)
+// and serves their table cells with the compiler-scheduled kernels.
+#ifdef SA_NO_ASM_KERNELS
+constexpr bool kAsmKernels = false;
+#else
+constexpr bool kAsmKernels = true;
+#endif
 inline LaunchChoice launch_choice(int D, int chunk, int back) {
   // head dimension 256 has one shape per kernel: anything wider or deeper does not fit registers or LDS
   if (D == 256) return LaunchChoice{FWD_NARROW, DQ_NARROW, DKDV_BLOCKSKIP};
   LaunchChoice c = (D == 128 ? TUNE_D128 : TUNE_D64)[chunk_class(chunk)][window_class(chunk, back)];
-  if (g_tune_override[0] >= 0 && g_tune_override[0] < FWD_VARIANTS) c.fwd = g_tune_override[0];
-  if (g_tune_override[1] >= 0 && g_tune_override[1] < DQ_VARIANTS) c.dq = g_tune_override[1];
-  if (g_tune_override[2] >= 0 && g_tune_override[2] < DKDV_VARIANTS) c.dkdv = g_tune_override[2];
-  if (D != 128 && c.dkdv == DKDV_PIPELINED) c.dkdv = DKDV_BLOCKSKIP;
-  if (D != 128 && c.dq == DQ_PIPELINED) c.dq = DQ_NARROW;
+  const int o0 = g_tune_override[0].load(std::memory_order_relaxed);
+  const int o1 = g_tune_override[1].load(std::memory_order_relaxed);
+  const int o2 = g_tune_override[2].load(std::memory_order_relaxed);
+  if (o0 >= 0 && o0 < FWD_VARIANTS) c.fwd = o0;
+  if (o1 >= 0 && o1 < DQ_VARIANTS) c.dq = o1;
+  if (o2 >= 0 && o2 < DKDV_VARIANTS) c.dkdv = o2;
+  const bool pipelined = kAsmKernels && D == 128;
+  if (!pipelined && c.dkdv == DKDV_PIPELINED) c.dkdv = DKDV_BLOCKSKIP;
+  if (!pipelined && c.dq == DQ_PIPELINED) c.dq = DQ_NARROW;
+  if (!pipelined && c.fwd == FWD_PIPELINED) c.fwd = FWD_NARROW;
   return c;
 }
 
 template <typename T> struct Cfg {
   static constexpr int NW = 4;                                   // waves per workgroup
-  // 16-bit, D in {64, 128, 256}: forward kernel with QB query blocks per wave and NST LDS stages
-  // The forward and dQ kernels come in two widths: 8 waves (256 queries) share each key tile among
-  // more waves, which pays once the workgroup's queries lie in one chunk; with smaller chunks the
-  // union of the waves' windows grows and 4 waves (128 queries) waste less of every tile.
-  static constexpr int WIDE_NW = 8, NARROW_NW = 4;
+  // 16-bit, D in {64, 128, 256}: forward kernel with QB query blocks per wave and NST LDS stages.
+  // The compiler-scheduled forward and dQ kernels run 4 waves (128 queries) per workgroup, two workgroups
+  // per CU (an 8-wave shape measured slower or equal in every cell of the tuning sweep and was removed).
+  static constexpr int NARROW_NW = 4;
   static constexpr int DQ2_TK = SA_DQ2_TK, DQ2_NST = SA_DQ2_NST;
   static constexpr int DKDV2_NW = SA_DKDV2_NW, DKDV2_TQ = SA_DKDV2_TQ, DKDV2_NST = SA_DKDV2_NST;
   // The software-pipelined dK/dV kernel exists at head dimension 128 only: at 64 a block step has

@@ -155,7 +155,7 @@ def test_every_kernel_variant_16bit(D, dtype):
     q, k, v, d_o = make_inputs(B, H, T, D, seed=32, dtype=dtype)
     lens = torch.tensor([T, 500], dtype=torch.int32)
     # pipelined variants exist at head dimension 128 only: (forward, dQ, dK/dV) variant ids per kernel
-    variants = ((0, 1), (0, 1, 2) if D == 128 else (0, 1), (0, 1, 2) if D == 128 else (0, 2))
+    variants = ((0, 1) if D == 128 else (0,), (0, 1) if D == 128 else (0,), (0, 1, 2) if D == 128 else (0, 2))
     try:
         for kernel in range(3):
             for variant in variants[kernel]:
@@ -301,7 +301,7 @@ def test_backward_op_reads_a_strided_forward_output(D, T, C, R):
     q, k, v, d_o = make_inputs(B, H, T, D, seed=33, dtype=dtype)
     lens = torch.tensor([T, T - 59], dtype=torch.int32)
     if D == 128:
-        assert _lib.load().sa_launch_choice(D, C, R, 1) == 2
+        assert _lib.load().sa_launch_choice(D, C, R, 1) == 1   # the software-pipelined dQ kernel
     qd, kd, vd = (t.to(dev) for t in (q, k, v))
     fwd = torch.ops.alexdremov_streaming_attention.forward
     bwd = torch.ops.alexdremov_streaming_attention.backward

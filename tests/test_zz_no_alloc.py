@@ -55,7 +55,7 @@ def test_static_backward_matches_workspace_backward_twice():
     _run_both(lib, _lib, 2, 2, 150, 64, 10, 3, torch.float32, 0, 42, [150, 77])
     _run_both(lib, _lib, 1, 2, 96, 64, 32, 1, torch.float16, 1, 43, None)
     # a window of 4608 keys at head dimension 128: the software-pipelined dQ and dK/dV kernels
-    assert lib.sa_launch_choice(128, 512, 8, 1) == 2 and lib.sa_launch_choice(128, 512, 8, 2) == 1
+    assert lib.sa_launch_choice(128, 512, 8, 1) == 1 and lib.sa_launch_choice(128, 512, 8, 2) == 1
     _run_both(lib, _lib, 1, 2, 5000, 128, 512, 8, torch.bfloat16, 2, 44, [4321])
 
 
