@@ -156,10 +156,6 @@ def time_kernels(w, iters, only=None):
     return out
 
 
-def time_kernels_only(w, iters, only):
-    return time_kernels(w, iters, only)
-
-
 def cpu_baseline(w, name, budget_s=12.0):
     """The CPU restatement of the algorithm timed on the host cores, on a bounded sample of the
     benchmarked workload: batch element 0 (all heads) through the chunk-by-chunk fp32 oracle,
@@ -207,15 +203,20 @@ def cpu_baseline(w, name, budget_s=12.0):
 
 # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (separate --pmc runs of this script, scaled by
 # what the same counters read for the 1 GiB copy of --calibrate-copy).  Counter runs cannot be made from
-# inside a timed run, so the figures of the committed summaries under profiles/ are quoted here; a
-# workload or kernel without a committed counter run reports null.
-HBM_BYTES_PER_LAUNCH = {
-    "headline_bf16_T16384_D128": {"fwd": 1.914e+09, "delta": 5.411e+08, "dq": 1.927e+09, "dkdv": 1.747e+09},
-    "bf16_T4096_D64": {"fwd": 3.072e+08, "delta": 1.364e+08, "dq": 4.847e+08, "dkdv": 5.352e+08},
-    "ragged_fp16_T2048_D128": {"fwd": 1.415e+08, "delta": 1.353e+08, "dq": 1.775e+08, "dkdv": 2.195e+08},
-    "long_bf16_T65536_D128": {"fwd": 1.378e+10, "delta": 1.082e+09, "dq": 8.672e+09, "dkdv": 5.757e+09},
-}
-TRAFFIC_SOURCE = "quoted from the rocprofv3 FETCH_SIZE/WRITE_SIZE summary under profiles/ (not measured in this run)"
+# inside a timed run, so the figures of the committed counter runs are quoted: profiles/hbm_traffic.json
+# holds them (the per-workload summaries under profiles/ show the same numbers with their commands;
+# tests/test_boundary.py checks that the two agree).  A workload or kernel without a counter run reports null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+TRAFFIC_SOURCE = "quoted from profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE/WRITE_SIZE runs; not measured in this run)"
+
+
+def hbm_bytes_per_launch():
+    """{workload: {kernel: HBM bytes per launch}} from the committed counter runs ({} if the file is missing)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            return json.load(f)["hbm_bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return {}
 
 
 def measured_ceilings():
@@ -380,6 +381,107 @@ def path_sweep(device, iters=10):
 
 
 
+VARIANT_NAMES = {"fwd": ["narrow", "pipelined"], "dq": ["narrow", "pipelined"], "dkdv": ["blockskip", "pipelined", "split"]}
+
+
+def measure_workload(name, dev, steps, warmup, kernel_iters, zeros=False, compiled=False):
+    """One workload: `steps` forward+backward steps through the public API between two synchronisations
+    (ms_per_step, value), the same step bracketed by events for the median (at least 50 of them), each
+    kernel on its own through the C ABI, and the roofline entry of the slowest kernel."""
+    import torch
+    from streaming_attention import _lib, compiled_wrapper, streaming_attention
+
+    w = make_inputs(name, dev, zeros=zeros)
+    B, H, T, D, C, R = w["B"], w["H"], w["T"], w["D"], w["C"], w["R"]
+    P = unmasked_pairs(T, C, R, w["lens_list"])
+    flops_step = 14.0 * D * H * P
+    q, k, v = (w[n].requires_grad_() for n in ("q", "k", "v"))
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        out = streaming_attention(q, k, v, w["lens"], C, R)
+        out.backward(w["d_o"])
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+    value = flops_step / (ms_per_step * 1e-3) / 1e12
+
+    # the same steps once more, each bracketed by events on the stream they run on, for the median
+    n_med = max(steps, 50)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_med)]
+    for e0, e1 in evs:
+        e0.record()
+        step()
+        e1.record()
+    torch.cuda.synchronize()
+    per_step = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+    median_ms = per_step[len(per_step) // 2] if len(per_step) % 2 else \
+        0.5 * (per_step[len(per_step) // 2 - 1] + per_step[len(per_step) // 2])
+
+    compiled_ms = None
+    if compiled:
+        # the same step through the torch.compile'd wrapper that the reference puts around the op
+        with compiled_wrapper():
+            for _ in range(warmup):
+                step()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            compiled_ms = (time.perf_counter() - t1) * 1e3 / steps
+
+    kt = time_kernels(w, kernel_iters)
+    lib = _lib.load()
+    variants = {kn: (VARIANT_NAMES[kn][lib.sa_launch_choice(D, C, R, ki)] if w["dtype"] != "float32" and D >= 64
+                     else "first generation")
+                for ki, kn in enumerate(("fwd", "dq", "dkdv"))}
+    # GEMMs each kernel performs per unmasked pair: fwd S,PV; dq S,dP,dQ; dkdv S,dP,dV,dK
+    kernel_flops = {"fwd": 4.0 * D * H * P, "dq": 6.0 * D * H * P, "dkdv": 8.0 * D * H * P}
+    es = 4 if w["dtype"] == "float32" else 2
+    N = B * H * T
+    tensor = float(N) * D * es
+    # Algorithmic HBM bytes per launch: every operand read once, every result written once.  Positions
+    # t >= lens[b] of the inputs are never read, the outputs are written in full (zeros there); delta
+    # reads all rows of O and dO.
+    valid = sum(min(int(L), T) for L in w["lens_list"]) / float(B * T)
+    rd, rows = tensor * valid, 4.0 * N
+    kernel_bytes = {"fwd": 3.0 * rd + tensor + rows, "delta": 2.0 * tensor + rows,
+                    "dq": 4.0 * rd + 2.0 * rows * valid + tensor, "dkdv": 4.0 * rd + 2.0 * rows * valid + 2.0 * tensor}
+    # per step every tensor once: forward reads q, k, v and writes O; backward reads q, k, v, O, dO and
+    # writes dQ, dK, dV; lse and delta are written and read once each
+    step_bytes = 8.0 * rd + 4.0 * tensor + 4.0 * rows
+    peak_tflops = PEAK_F32_TFLOPS if w["dtype"] == "float32" else PEAK_BF16_TFLOPS
+    balance = peak_tflops * 1e12 / (PEAK_HBM_GBS * 1e9)            # flop per byte at which the two roofs meet
+    intensity = flops_step / step_bytes
+    bound = "mfma" if intensity >= balance else "hbm"
+    dom = max(kernel_flops, key=lambda n: kt[n])
+    traffic = hbm_bytes_per_launch().get(name, {}).get(dom)
+    if bound == "mfma":
+        achieved = kernel_flops[dom] / (kt[dom] * 1e-3) / 1e12
+        roofline = {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": peak_tflops, "unit": "TFLOP/s",
+                    "frac": achieved / peak_tflops}
+    else:
+        achieved = kernel_bytes[dom] / (kt[dom] * 1e-3) / 1e9
+        roofline = {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": achieved / PEAK_HBM_GBS}
+    roofline.update({"traffic": traffic, "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
+                     "algorithmic_bytes": kernel_bytes[dom], "algorithmic_flops": kernel_flops[dom],
+                     "arithmetic_intensity_flop_per_byte": intensity, "machine_balance_flop_per_byte": balance})
+    q.grad = k.grad = v.grad = None
+    return {"inputs": w, "pairs": P, "flops_step": flops_step, "step_bytes": step_bytes, "ms_per_step": ms_per_step,
+            "value": value, "median_ms": median_ms, "median_steps": n_med, "compiled_wrapper_ms_per_step": compiled_ms,
+            "kernel_ms": kt, "kernel_variants": variants,
+            "kernel_tflops": {n: kernel_flops[n] / (kt[n] * 1e-3) / 1e12 for n in kernel_flops},
+            "kernel_gbs": {n: kernel_bytes[n] / (kt[n] * 1e-3) / 1e9 for n in kernel_bytes}, "roofline": roofline}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -388,6 +490,8 @@ def main():
     ap.add_argument("--workload", default=DEFAULT, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the MFMA / copy ceiling measurement")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="with the default workload: do not time the other GPU configurations after it")
     ap.add_argument("--kernel-iters", type=int, default=10)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy (known traffic) for scaling HBM counters")
@@ -405,7 +509,6 @@ def main():
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
 
     import torch
-    from streaming_attention import streaming_attention
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
@@ -429,112 +532,63 @@ def main():
         print(json.dumps({"sweep": "kernel variants, B=4 H=16 T=16384, lens ~ U[T/2, T]", "n_gpus": 1,
                           "rows": tune_sweep(dev)}))
         return
-    w = make_inputs(args.workload, dev, zeros=args.zero_inputs)
+    m = measure_workload(args.workload, dev, args.steps, args.warmup, args.kernel_iters, zeros=args.zero_inputs,
+                         compiled=True)
+    w, kt = m["inputs"], m["kernel_ms"]
     B, H, T, D, C, R = w["B"], w["H"], w["T"], w["D"], w["C"], w["R"]
-    P = unmasked_pairs(T, C, R, w["lens_list"])
-    flops_step = 14.0 * D * H * P
-    q, k, v = (w[n].requires_grad_() for n in ("q", "k", "v"))
-
-    def step():
-        q.grad = k.grad = v.grad = None
-        out = streaming_attention(q, k, v, w["lens"], C, R)
-        out.backward(w["d_o"])
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    value = flops_step / (ms_per_step * 1e-3) / 1e12
-
-    # the same steps once more, each bracketed by events on the stream they run on, for the median
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    for e0, e1 in evs:
-        e0.record()
-        step()
-        e1.record()
-    torch.cuda.synchronize()
-    per_step = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
-    median_ms = per_step[len(per_step) // 2] if len(per_step) % 2 else \
-        0.5 * (per_step[len(per_step) // 2 - 1] + per_step[len(per_step) // 2])
-
-    # the same step through the torch.compile'd wrapper that the reference puts around the op
-    os.environ["STREAMING_ATTENTION_COMPILED"] = "1"
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    compiled_wrapper_ms_per_step = (time.perf_counter() - t1) * 1e3 / args.steps
-    os.environ.pop("STREAMING_ATTENTION_COMPILED", None)
-
-    kt = time_kernels(w, args.kernel_iters)
-    # GEMMs each kernel performs per unmasked pair: fwd S,PV; dq S,dP,dQ; dkdv S,dP,dV,dK
-    kernel_flops = {"fwd": 4.0 * D * H * P, "dq": 6.0 * D * H * P, "dkdv": 8.0 * D * H * P}
-    es = 4 if w["dtype"] == "float32" else 2
-    N = B * H * T
-    tensor = float(N) * D * es
-    # Algorithmic HBM bytes per launch: every operand read once, every result written once.  Positions
-    # t >= lens[b] of the inputs are never read, the outputs are written in full (zeros there); delta
-    # reads all rows of O and dO.
-    valid = sum(min(int(L), T) for L in w["lens_list"]) / float(B * T)
-    rd, rows = tensor * valid, 4.0 * N
-    kernel_bytes = {"fwd": 3.0 * rd + tensor + rows, "delta": 2.0 * tensor + rows,
-                    "dq": 4.0 * rd + 2.0 * rows * valid + tensor, "dkdv": 4.0 * rd + 2.0 * rows * valid + 2.0 * tensor}
-    # per step every tensor once: forward reads q, k, v and writes O; backward reads q, k, v, O, dO and
-    # writes dQ, dK, dV; lse and delta are written and read once each
-    step_bytes = 8.0 * rd + 4.0 * tensor + 4.0 * rows
-    peak_tflops = PEAK_F32_TFLOPS if w["dtype"] == "float32" else PEAK_BF16_TFLOPS
-    balance = peak_tflops * 1e12 / (PEAK_HBM_GBS * 1e9)            # flop per byte at which the two roofs meet
-    intensity = flops_step / step_bytes
-    bound = "mfma" if intensity >= balance else "hbm"
-    dom = max(kernel_flops, key=lambda n: kt[n])
-    traffic = HBM_BYTES_PER_LAUNCH.get(args.workload, {}).get(dom)
-    if bound == "mfma":
-        achieved = kernel_flops[dom] / (kt[dom] * 1e-3) / 1e12
-        roofline = {"kernel": dom, "bound": "mfma", "achieved": achieved, "peak": peak_tflops, "unit": "TFLOP/s",
-                    "frac": achieved / peak_tflops}
-    else:
-        achieved = kernel_bytes[dom] / (kt[dom] * 1e-3) / 1e9
-        roofline = {"kernel": dom, "bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": achieved / PEAK_HBM_GBS}
-    roofline.update({"traffic": traffic, "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
-                     "algorithmic_bytes": kernel_bytes[dom], "algorithmic_flops": kernel_flops[dom],
-                     "arithmetic_intensity_flop_per_byte": intensity, "machine_balance_flop_per_byte": balance})
     P_blocks = unmasked_block_pairs(T, C, R, w["lens_list"])
     result = {
         "metric": "effective TFLOP/s fwd+bwd (unmasked blocks) at 1 GPU; % of bf16 MFMA peak",
-        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "median_ms": median_ms, "compiled_wrapper_ms_per_step": compiled_wrapper_ms_per_step,
+        "value": m["value"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": m["ms_per_step"], "median_ms": m["median_ms"], "median_steps": m["median_steps"],
+        "compiled_wrapper_ms_per_step": m["compiled_wrapper_ms_per_step"],
         "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None,
         "dtype": {"bfloat16": "bf16", "float16": "f16", "float32": "f32"}[w["dtype"]],
         "data": "synthetic, all zeros (diagnostic run)" if args.zero_inputs else "synthetic",
         "config": {"workload": args.workload, "B": B, "H": H, "T": T, "D": D, "context_size": C,
-                   "back_contexts": R, "lens": w["lens_list"], "unmasked_pairs_per_head": P,
-                   "flops_per_step": flops_step, "algorithmic_bytes_per_step": step_bytes},
-        "pct_of_bf16_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
-        "value_block_granular": 14.0 * D * H * P_blocks / (ms_per_step * 1e-3) / 1e12,
-        "step_hbm_gbs": step_bytes / (ms_per_step * 1e-3) / 1e9,
+                   "back_contexts": R, "lens": w["lens_list"], "unmasked_pairs_per_head": m["pairs"],
+                   "flops_per_step": m["flops_step"], "algorithmic_bytes_per_step": m["step_bytes"]},
+        "pct_of_bf16_mfma_peak": 100.0 * m["value"] / PEAK_BF16_TFLOPS,
+        "value_block_granular": 14.0 * D * H * P_blocks / (m["ms_per_step"] * 1e-3) / 1e12,
+        "step_hbm_gbs": m["step_bytes"] / (m["ms_per_step"] * 1e-3) / 1e9,
         "peaks_used": {"bf16_mfma_tflops": PEAK_BF16_TFLOPS, "f32_mfma_tflops": PEAK_F32_TFLOPS,
                        "hbm_gbs": PEAK_HBM_GBS},
         "kernel_ms": kt,
+        "kernel_variants": m["kernel_variants"],
         "kernel_ms_note": ("each kernel launched on its own through the C ABI; for this dtype and head dimension the step's "
                            "backward forms delta inside the dQ kernel and does not launch the delta pass timed here"
                            if w["dtype"] != "float32" and D >= 64 else "each kernel launched on its own through the C ABI"),
-        "kernel_tflops": {n: kernel_flops[n] / (kt[n] * 1e-3) / 1e12 for n in kernel_flops},
-        "kernel_gbs": {n: kernel_bytes[n] / (kt[n] * 1e-3) / 1e9 for n in kernel_bytes},
-        "roofline": roofline,
+        "kernel_tflops": m["kernel_tflops"],
+        "kernel_gbs": m["kernel_gbs"],
+        "roofline": m["roofline"],
     }
+    del w, m
+    torch.cuda.empty_cache()
+    if args.workload == DEFAULT and not args.zero_inputs and not args.no_other_workloads:
+        # the other GPU configurations of the baseline, timed after the headline (which stays `value`):
+        # fewer steps where a step is long, more where the host would otherwise dominate
+        others = {}
+        for name, steps in (("bf16_T4096_D64", 200), ("ragged_fp16_T2048_D128", 300), ("long_bf16_T65536_D128", 10)):
+            o = measure_workload(name, dev, steps, 5, args.kernel_iters if "long" not in name else 3)
+            dom = o["roofline"]["kernel"]
+            others[name] = {
+                "ms_per_step": o["ms_per_step"], "median_ms": o["median_ms"], "steps": steps,
+                "effective_tflops": o["value"], "pct_of_bf16_mfma_peak": 100.0 * o["value"] / PEAK_BF16_TFLOPS,
+                "step_hbm_gbs": o["step_bytes"] / (o["ms_per_step"] * 1e-3) / 1e9,
+                "kernel_ms": o["kernel_ms"], "kernel_variants": o["kernel_variants"], "dominant_kernel": dom,
+                "roofline": {k: o["roofline"][k] for k in ("kernel", "bound", "achieved", "peak", "unit", "frac", "traffic")},
+                "config": {"B": o["inputs"]["B"], "H": o["inputs"]["H"], "T": o["inputs"]["T"], "D": o["inputs"]["D"],
+                           "dtype": o["inputs"]["dtype"], "context_size": o["inputs"]["C"],
+                           "back_contexts": o["inputs"]["R"], "lens": o["inputs"]["lens_list"]},
+            }
+            del o
+            torch.cuda.empty_cache()
+        result["other_workloads"] = others
     if not args.no_ceilings:
         result["measured_ceilings"] = measured_ceilings()
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(w, args.workload)
+        result["cpu_baseline"] = cpu_baseline(make_inputs(args.workload, dev, zeros=args.zero_inputs), args.workload)
     print(json.dumps(result))
 
 

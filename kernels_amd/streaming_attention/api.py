@@ -1,7 +1,9 @@
 """Public functions, signature-compatible with src/streaming_attention/kernel.py:1533-1652."""
 from __future__ import annotations
 
+import contextlib
 import os
+import threading
 
 import torch
 import torch.nn.functional as F
@@ -47,6 +49,33 @@ def _forward_op(q, k, v, lens, context_size, back_contexts, sm_scale, autotune, 
 
 
 _compiled = None
+_call_path = threading.local()
+
+
+@contextlib.contextmanager
+def compiled_wrapper(enabled: bool = True):
+    """Route the calls of ``streaming_attention`` made inside the ``with`` block (on this thread) through the
+    ``torch.compile(fullgraph=True, dynamic=True)`` wrapper that the reference puts around every call
+    (kernel.py:1566-1596), or, with ``enabled=False``, straight to the op whatever the environment says.
+    Results are identical either way; the wrapper costs guard checks per call."""
+    previous = getattr(_call_path, "compiled", None)
+    _call_path.compiled = bool(enabled)
+    try:
+        yield
+    finally:
+        _call_path.compiled = previous
+
+
+def _use_compiled_wrapper() -> bool:
+    """Which path a call takes: the ``compiled_wrapper`` context of this thread if one is active, else
+    ``STREAMING_ATTENTION_COMPILED=1`` (wrapper) or ``STREAMING_ATTENTION_EAGER=0`` (wrapper; ``=1`` names the
+    default), else the direct op call."""
+    scoped = getattr(_call_path, "compiled", None)
+    if scoped is not None:
+        return scoped
+    if os.environ.get("STREAMING_ATTENTION_COMPILED") == "1":
+        return True
+    return os.environ.get("STREAMING_ATTENTION_EAGER") == "0"
 
 
 def _compiled_forward():
@@ -90,7 +119,8 @@ def streaming_attention(
 
     The op is called directly.  The reference routes every call through a
     ``torch.compile(fullgraph=True, dynamic=True)`` wrapper (kernel.py:1566-1596); that wrapper is
-    kept and runs when ``STREAMING_ATTENTION_COMPILED=1`` is set, but it is not the default: the
+    kept and runs inside ``with compiled_wrapper():`` (per call site) or when
+    ``STREAMING_ATTENTION_COMPILED=1`` is set (process-wide), but it is not the default: the
     graph it holds is this one opaque op, so it changes no result, and its guard checks and
     AOTAutograd wrappers cost about 0.1 ms of host time per forward+backward, as much as all four
     kernels of a small problem take on the GPU.
@@ -102,7 +132,7 @@ def streaming_attention(
         sm_scale=sm_scale, autotune=autotune, return_lse=return_lse, prescale_qk=prescale_qk,
         precision=precision,
     )
-    if torch.compiler.is_compiling() or os.environ.get("STREAMING_ATTENTION_COMPILED") != "1":
+    if torch.compiler.is_compiling() or not _use_compiled_wrapper():
         return _forward_op(**args)
     for t in (q, k, v):
         torch._dynamo.mark_static(t, 1)

@@ -5,7 +5,11 @@ the reference (src/streaming_attention/kernel.py:1270-1530); the bodies enqueue 
 kernels of libstreaming_attention.so on the current stream instead of launching Triton
 kernels.  ``autotune``, ``prescale_qk`` and ``precision`` are accepted for signature
 compatibility and do not change the result: kernel variants are read from a table measured
-on MI355X (head dimension, context_size class, window class) and all accumulation is fp32.
+on MI355X (head dimension, context_size class, window class), all accumulation is fp32, and
+where the scale is applied is fixed per kernel: in float32 inside the exp2 argument in the forward
+and dQ kernels (at least as accurate as either setting of ``prescale_qk``), folded into K and
+rounded to the element type in the 16-bit dK/dV kernels at head dimensions 64 and up (what the
+reference does under ``prescale_qk=True``, kernel.py:1065-1066).
 """
 from __future__ import annotations
 
@@ -293,3 +297,33 @@ class _StreamingAttention(torch.autograd.Function):
 
 
 _LIBRARY.impl("forward", _StreamingAttention.apply, "Autograd")
+
+
+class _NoDoubleBackward(torch.autograd.Function):
+    """Marks the outputs of the backward op as not differentiable a second time: the reference registers
+    no autograd formula for ``::backward`` (kernel.py:1360-1442), so differentiating through it raises
+    there; it raises here as well instead of silently returning detached gradients."""
+
+    @staticmethod
+    def forward(ctx, dq, dk, dv, *inputs):
+        return dq.view_as(dq), dk.view_as(dk), dv.view_as(dv)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise RuntimeError(
+            "alexdremov_streaming_attention::backward has no autograd formula: "
+            "differentiating through the backward pass (double backward) is not supported")
+
+
+def _backward_autograd(q, k, v, lens, o, lse, do, context_size, back_contexts, sm_scale, autotune,
+                       prescale_qk, precision):
+    with torch._C._AutoDispatchBelowAutograd():
+        DQ, DK, DV = torch.ops.alexdremov_streaming_attention.backward(
+            q, k, v, lens, o, lse, do, context_size, back_contexts, sm_scale, autotune, prescale_qk, precision)
+    # under an ordinary .backward() gradient mode is off and nothing is recorded
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v, o, do)):
+        return _NoDoubleBackward.apply(DQ, DK, DV, q, k, v, o, do)
+    return DQ, DK, DV
+
+
+_LIBRARY.impl("backward", _backward_autograd, "Autograd")

@@ -75,7 +75,8 @@ def unmasked_pairs(T: int, context_size: int, back_contexts: int, L) -> int:
     return total
 
 
-def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=None, round_dtype=None):
+def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=None, round_dtype=None,
+              prescaled_k=False):
     """Explicit float64 evaluation.  Returns dict with O, LSE (log2 units, 0 at padded
     rows) and, when ``d_out`` is given, dQ, dK, dV (all numpy float64).
 
@@ -83,7 +84,11 @@ def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=N
     a 16-bit kernel must evaluate them: the probabilities and dS are rounded to that type before
     the second matrix products (the reference does the same: kernel.py:370, 1020, 1121, 1127), the
     softmax denominator sums the rounded probabilities, and O is rounded before delta is formed.
-    The difference between the two evaluations is the error that rounding alone causes."""
+    The difference between the two evaluations is the error that rounding alone causes.
+    ``prescaled_k`` (with ``round_dtype``) also models the scores of the 16-bit dK/dV kernels for head
+    dimensions 64 and up, which fold -scale*log2(e) into K and round the product to the element type
+    before the score product (the reference's prescale_qk=True, kernel.py:1065-1066): dK and dV are then
+    formed from probabilities exp2(q . round(k*scale*log2e) - lse), dQ from the unrounded scale."""
     qn, kn, vn = (t.detach().cpu().double() for t in (q, k, v))
     B, H, T, D = qn.shape
     s = float(D) ** -0.5 if sm_scale is None else float(sm_scale)
@@ -118,10 +123,15 @@ def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=N
         delta = (Ob * g).sum(-1, keepdim=True)
         dP = torch.matmul(g, vn.transpose(-1, -2))
         dS = Pb * (dP - delta)
-        Pb, dS = rounded(Pb), rounded(dS)
-        out["dV"] = torch.matmul(Pb.transpose(-1, -2), g).numpy()
+        Pkv, dSkv = Pb, dS
+        if round_dtype is not None and prescaled_k:
+            S2 = torch.matmul(qn, rounded(kn * (s * LOG2E)).transpose(-1, -2))           # log2 units
+            Pkv = torch.where(mask, torch.exp2(S2 - lse[..., None]), 0.0) * row_valid
+            dSkv = Pkv * (dP - delta)
+        Pkv, dS, dSkv = rounded(Pkv), rounded(dS), rounded(dSkv)
+        out["dV"] = torch.matmul(Pkv.transpose(-1, -2), g).numpy()
         out["dQ"] = (s * torch.matmul(dS, kn)).numpy()
-        out["dK"] = (s * torch.matmul(dS.transpose(-1, -2), qn)).numpy()
+        out["dK"] = (s * torch.matmul(dSkv.transpose(-1, -2), qn)).numpy()
     return out
 
 

@@ -9,11 +9,10 @@ import torch
 TOL = {torch.float32: (1e-4, 0.0), torch.float16: (2e-2, 1e-2), torch.bfloat16: (2e-2, 1e-2)}
 
 
-# The log-sum-exp is a float32 output whatever the input type.  For 16-bit inputs the kernels sum the
-# ROUNDED probabilities (the weights the PV product really applies, so that they add up to one): the
-# relative error of that sum is at most the unit roundoff u of the type, i.e. at most log2(e) * u in
-# the base-2 logarithm: 7.0e-4 for float16 (u = 2^-11), 5.6e-3 for bfloat16 (u = 2^-8).
-LSE_ATOL = {torch.float32: 1e-4, torch.float16: 1e-3, torch.bfloat16: 6e-3}
+# The log-sum-exp is a float32 output whatever the input type: scores are accumulated in float32 from the
+# (exactly representable) 16-bit inputs, scaled in float32, and the probabilities are summed in float32
+# before they are rounded for the second product, so the bar is the float32 one for every type.
+LSE_ATOL = {torch.float32: 1e-4, torch.float16: 1e-4, torch.bfloat16: 1e-4}
 
 
 def make_inputs(B, H, T, D, seed=20, dtype=torch.float32):
@@ -69,17 +68,20 @@ def error_report(got, want):
 
 def assert_close_rounding_aware(name, got, exact, rounded, dtype):
     """The BASELINE bar widened by the error that rounding P and dS to ``dtype`` causes in a
-    float64 evaluation of the same formulas: bound = atol + rtol * |exact| + 2 * max |rounded - exact|.
-    Individual rounding errors are random, so the allowance is the largest deviation anywhere in the
-    tensor, not the deviation of the same element."""
+    float64 evaluation of the same formulas: bound = atol + rtol * |exact| + 2 * max |rounded - exact|,
+    the maximum taken over the element's own (batch, head) slice.  The allowance cannot be narrower than
+    that: the largest part of a row's deviation is one random number per row (the error of delta, which
+    multiplies the whole row of dS), so a single row of the float64 evaluation says little about the same
+    row of another evaluation with other rounding errors, while the rows of one head are samples of the
+    same distribution.  A wrong element in another head or batch entry gets no cover from it."""
     atol, rtol = TOL[dtype]
     got = torch.as_tensor(got).detach().double().cpu()
     exact = torch.as_tensor(exact).detach().double().cpu()
     rounded = torch.as_tensor(rounded).detach().double().cpu()
     assert torch.isfinite(got).all(), f"{name}: non-finite values"
-    allowance = 2.0 * (rounded - exact).abs().max().item()
+    allowance = 2.0 * (rounded - exact).abs().amax((-2, -1), keepdim=True)
     err = (got - exact).abs()
     bad = err > atol + rtol * exact.abs() + allowance
     assert not bad.any(), (
         f"{name}: {int(bad.sum())} elements out of tolerance, max abs err {err.max().item():.3e} "
-        f"(atol {atol}, rtol {rtol}, rounding allowance {allowance:.3e})")
+        f"(atol {atol}, rtol {rtol}, largest per-head rounding allowance {allowance.max().item():.3e})")

@@ -225,3 +225,34 @@ def test_flop_counter_matches_oracle():
 
     for T, C, R, lens in ((512, 64, 2, [300, 512]), (100, 7, 3, [1, 99, 100]), (64, 1000, 0, [64])):
         assert bench.unmasked_pairs(T, C, R, lens) == sa_oracle.unmasked_pairs(T, C, R, lens)
+
+
+def test_traffic_figures_match_profile_summaries():
+    """`roofline.traffic` is quoted from profiles/hbm_traffic.json; every figure in it must be the
+    'HBM bytes / launch' entry of the traffic table in the per-workload summary it is said to come from."""
+    sys.path.insert(0, ROOT)
+    import bench
+
+    summaries = {
+        "headline_bf16_T16384_D128": "streaming_attention_bf16_B4_H16_T16384_D128_C256_R8.md",
+        "bf16_T4096_D64": "streaming_attention_bf16_B8_H16_T4096_D64_C128_R4.md",
+        "ragged_fp16_T2048_D128": "streaming_attention_fp16_B16_H8_T2048_D128_C64_R1_ragged.md",
+        "long_bf16_T65536_D128": "streaming_attention_bf16_B1_H32_T65536_D128_C512_R16.md",
+    }
+    quoted = bench.hbm_bytes_per_launch()
+    assert set(quoted) == set(summaries)
+    for workload, fname in summaries.items():
+        text = open(os.path.join(ROOT, "profiles", fname)).read()
+        section = text[text.index("## 2. HBM traffic"):text.index("## 3.")]
+        header = next(ln for ln in section.splitlines() if ln.startswith("| kernel |"))
+        col = [c.strip() for c in header.strip("|").split("|")].index("HBM bytes / launch")
+        table = {}
+        for ln in section.splitlines():
+            cells = [c.strip() for c in ln.strip("|").split("|")]
+            if ln.startswith("|") and len(cells) > col and cells[0] not in ("kernel", "---"):
+                # fwd2 / fwd3 -> fwd, dq2 / dq3 -> dq, dkdv2 / dkdv3 / dkdv_split -> dkdv, delta
+                table[re.sub(r"(_split|\d)+$", "", cells[0])] = float(cells[col])
+        assert set(quoted[workload]) == set(table) == {"fwd", "dq", "dkdv", "delta"}, workload
+        for kernel, value in quoted[workload].items():
+            assert value == pytest.approx(table[kernel], rel=1e-9), (workload, kernel)
+    assert set(quoted) <= set(bench.WORKLOADS)

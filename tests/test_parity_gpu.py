@@ -81,18 +81,22 @@ def strided_gradient_and_lens(d_o, lens):
     return g, ld
 
 
-@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+# (dtype, noncontiguous): the reference's grid has float32 and float16 on both settings of its
+# "noncontiguous" axis and no bfloat16 at all; bfloat16 is added here on the contiguous setting
+DTYPE_LAYOUTS = [(torch.float32, False), (torch.float32, True), (torch.float16, False), (torch.float16, True),
+                 (torch.bfloat16, False)]
+
+
+@pytest.mark.parametrize("dtype,noncontiguous", DTYPE_LAYOUTS, ids=lambda x: str(x))
 @pytest.mark.parametrize("D", [16, 64])
 @pytest.mark.parametrize("lens_mode", ["none", "tricky"])
-@pytest.mark.parametrize("noncontiguous", [False, True])
 @pytest.mark.parametrize("C,R", WINDOWS)
 @pytest.mark.parametrize("B,H,T", SHAPES)
 def test_reference_grid(B, H, T, D, C, R, noncontiguous, lens_mode, dtype):
     """The reference's own grid (tests/test_streaming_attention.py:11-31), reduced: batch 40 and 6
-    heads at the short lengths, the long length at batch 5, and its strided float32 upstream gradient
-    and strided lens on every "noncontiguous" case (float32 and float16, as there)."""
-    if noncontiguous and dtype == torch.bfloat16:
-        pytest.skip("the reference's grid has no bfloat16 axis; covered by the contiguous case")
+    heads at the short lengths, the long length at batch 5 (test_reference_grid_full_batch runs it at
+    batch 40 with 6 heads), and its strided float32 upstream gradient and strided lens on every
+    "noncontiguous" case (float32 and float16, as there)."""
     q, k, v, d_o = make_inputs(B, H, T, D, dtype=dtype)
     lens = tricky_lens(B, T, C, R) if lens_mode == "tricky" else None
     if not noncontiguous:
@@ -108,6 +112,33 @@ def test_reference_grid(B, H, T, D, C, R, noncontiguous, lens_mode, dtype):
     ref = sa_oracle.dense_f64(q, k, v, lens, C, R, d_out=d_o)
     for name, got in (("O", out), ("dQ", qd.grad), ("dK", kd.grad), ("dV", vd.grad)):
         assert_close(name, got, ref[name], dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=str)
+@pytest.mark.parametrize("D", [16, 64])
+@pytest.mark.parametrize("lens_mode", ["none", "tricky"])
+@pytest.mark.parametrize("C,R", [(1, 5), (10, 0), (10, 5), (32, 5), (10000, 10000)])
+def test_reference_grid_full_batch(C, R, lens_mode, D, dtype):
+    """The largest cell of the reference's grid at its real size (batch 40, 6 heads, T = 800,
+    tests/test_streaming_attention.py:26-28), compared the way the reference's test compares: against
+    dense-mask SDPA evaluated in float32 on the same GPU (tests/test_streaming_attention.py:152-222),
+    which is the oracle's `sdpa_fwd_bwd` formulation."""
+    from streaming_attention import streaming_attention
+
+    B, H, T = 40, 6, 800
+    dev = torch.device("cuda:0")
+    q, k, v, d_o = (t.to(dev) for t in make_inputs(B, H, T, D, dtype=dtype))
+    lens = tricky_lens(B, T, C, R).to(dev) if lens_mode == "tricky" else None
+    qd, kd, vd = (t.clone().requires_grad_() for t in (q, k, v))
+    out = streaming_attention(qd, kd, vd, lens, C, R)
+    out.backward(d_o)
+    want = sa_oracle.sdpa_fwd_bwd(q, k, v, lens, C, R, d_o)
+    for name, got, ref in zip(("O", "dQ", "dK", "dV"), (out, qd.grad, kd.grad, vd.grad), want):
+        got, ref = got.detach().float(), ref.float()
+        atol, rtol = TOL[dtype]
+        assert torch.isfinite(got).all(), name
+        bad = (got - ref).abs() > atol + rtol * ref.abs()
+        assert not bool(bad.any()), f"{name}: {int(bad.sum())} elements out of tolerance, max {(got - ref).abs().max().item():.3e}"
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=str)
@@ -323,7 +354,8 @@ def check_rounding_aware(q, k, v, d_o, lens, C, R, dtype, sm_scale=None, record=
     kw = {} if sm_scale is None else {"sm_scale": sm_scale}
     o, lse, dq, dk, dv = run_kernel(q, k, v, d_o, lens, C, R, **kw)
     exact = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=sm_scale, d_out=d_o)
-    rounded = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=sm_scale, d_out=d_o, round_dtype=dtype)
+    rounded = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=sm_scale, d_out=d_o, round_dtype=dtype,
+                                  prescaled_k=q.shape[-1] >= 64)
     for name, got in (("O", o), ("dQ", dq), ("dK", dk), ("dV", dv)):
         assert_close_rounding_aware(name, got, exact[name], rounded[name], dtype)
         mx, rel, fro = error_report(got, exact[name])
@@ -421,15 +453,65 @@ def test_random_problems(seed):
     out.backward(d_o.to(dev))
     ref = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=scale, d_out=d_o)
     assert_close_lse(lse, ref["LSE"], dtype)
-    if dtype == torch.float32:
-        for name, got in (("O", out), ("dQ", qd.grad), ("dK", kd.grad), ("dV", vd.grad)):
+    results = (("O", out), ("dQ", qd.grad), ("dK", kd.grad), ("dV", vd.grad))
+    if dtype == torch.float32 or scale is None:
+        # the plain bar: 1e-4 for float32, 2e-2 + 1e-2 |ref| for the 16-bit types
+        for name, got in results:
             assert_close(name, got, ref[name], dtype)
     else:
         # explicit scales up to 0.2 at head dimensions up to 256 give scores of standard deviation 3:
-        # the bar allows for the rounding of P and dS (see check_rounding_aware)
-        rnd = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=scale, d_out=d_o, round_dtype=dtype)
-        for name, got in (("O", out), ("dQ", qd.grad), ("dK", kd.grad), ("dV", vd.grad)):
+        # the bar allows for the rounding of P and dS, and of the pre-scaled K in the dK/dV kernels,
+        # as a float64 evaluation with those roundings shows it (see check_rounding_aware)
+        rnd = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=scale, d_out=d_o, round_dtype=dtype,
+                                  prescaled_k=D >= 64)
+        for name, got in results:
             assert_close_rounding_aware(name, got, ref[name], rnd[name], dtype)
+    if dtype != torch.float32:
+        for name, got in results:
+            fro = error_report(got, ref[name])[2]
+            assert fro <= (2e-2 if dtype == torch.bfloat16 else 4e-3), f"{name}: relative Frobenius error {fro:.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("scale,q_gain", [(0.2, 1.0), (0.37, 1.0), (None, 6.0)])
+def test_pinned_variants_large_scores(scale, q_gain, dtype, capsys):
+    """Every forward, dQ and dK/dV variant at head dimension 128 pinned in turn on scores far from the
+    default: explicit scales 0.2 and 0.37 (standard deviation 3.3 and 6 in base-2 units) and, with the
+    default scale, queries multiplied by 6 (scores of standard deviation 8.7, maxima around 35-45 in
+    base-2 units).  The dK/dV kernels rebuild their probabilities from K pre-multiplied by
+    -scale*log2(e) and rounded to the element type, one more rounding than the forward pass makes;
+    the bound is the plain bar plus what a float64 evaluation with exactly those roundings deviates
+    from the exact one, head by head.  The margins are printed (pytest -s shows them)."""
+    from streaming_attention import _lib
+
+    lib = _lib.load()
+    B, H, T, D, C, R = 2, 2, 600, 128, 128, 2
+    q, k, v, d_o = make_inputs(B, H, T, D, seed=61, dtype=dtype)
+    q = (q.float() * q_gain).to(dtype)
+    lens = torch.tensor([T, 389], dtype=torch.int32)
+    exact = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=scale, d_out=d_o)
+    rounded = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=scale, d_out=d_o, round_dtype=dtype, prescaled_k=True)
+    kw = {} if scale is None else {"sm_scale": scale}
+    lines = []
+    try:
+        for kernel, name, variants in ((0, "fwd", (0, 1)), (1, "dq", (0, 1)), (2, "dkdv", (0, 1, 2))):
+            for variant in variants:
+                assert lib.sa_tune_override(kernel, variant) == 0
+                assert lib.sa_launch_choice(D, C, R, kernel) == variant
+                o, lse, dq, dk, dv = run_kernel(q, k, v, d_o, lens, C, R, **kw)
+                assert_close_lse(lse, exact["LSE"], dtype)
+                for tname, got in (("O", o), ("dQ", dq), ("dK", dk), ("dV", dv)):
+                    assert_close_rounding_aware(tname, got, exact[tname], rounded[tname], dtype)
+                    mx, _, fro = error_report(got, exact[tname])
+                    ref_t = torch.from_numpy(exact[tname])
+                    plain = (got.double() - ref_t).abs() - (TOL[dtype][0] + TOL[dtype][1] * ref_t.abs())
+                    lines.append(f"{name}={variant} {tname}: max abs {mx:.2e}, Frobenius {fro:.2e}, over the plain bar by {max(plain.max().item(), 0.0):.2e}")
+            assert lib.sa_tune_override(kernel, -1) == 0
+    finally:
+        for kernel in range(3):
+            lib.sa_tune_override(kernel, -1)
+    with capsys.disabled():
+        print(f"\n[pinned variants] {dtype} scale {scale} q x {q_gain}: max |LSE| {np.abs(exact['LSE']).max():.1f}\n  " + "\n  ".join(lines))
 
 
 @pytest.mark.parametrize("dtype,D", [(torch.float32, 64), (torch.bfloat16, 128), (torch.float16, 256)])

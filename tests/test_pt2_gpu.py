@@ -42,30 +42,82 @@ def test_opcheck(dtype, use_lens):
 
 
 @pytest.mark.parametrize("lens_mode", ["none", "random"])
-def test_compiled_wrapper_does_not_recompile_per_shape(lens_mode, monkeypatch):
-    monkeypatch.setenv("STREAMING_ATTENTION_COMPILED", "1")
-    from streaming_attention import streaming_attention
+def test_compiled_wrapper_does_not_recompile_per_shape(lens_mode):
+    """The reference's dynamic-shape sweep at its own size (tests/test_streaming_attention.py:271-310):
+    32 x 32 (batch, time) sizes up to 993 x 993 through the compiled wrapper, at most 4 graphs."""
+    from streaming_attention import compiled_wrapper, streaming_attention
 
     torch._dynamo.reset()
     torch._dynamo.utils.counters["stats"].clear()
     dev = torch.device("cuda:0")
     torch.empty(1, device=dev, requires_grad=True).backward()
     H, D = 4, 32
-    g = torch.Generator().manual_seed(31)
-    for B in range(1, 200, 48):
-        for T in range(1, 400, 96):
-            q, k, v = [torch.randn(B, H, T, D, generator=g).to(torch.float16).to(dev).requires_grad_() for _ in range(3)]
-            lens = None
-            if lens_mode == "random":
-                lens = torch.randint(1, T + 1, (B,), generator=g, dtype=torch.int32).to(dev)
-            out = streaming_attention(q, k, v, lens, context_size=16, back_contexts=2)
-            out.backward(torch.randn_like(out))
-            assert torch._dynamo.utils.counters["stats"]["unique_graphs"] <= 4
+    g = torch.Generator(device=dev).manual_seed(31)
+    with compiled_wrapper():
+        for B in range(1, 1024, 32):
+            for T in range(1, 1024, 32):
+                q, k, v = [((torch.rand(B, H, T, D, generator=g, device=dev) - 0.5) * 0.02).to(torch.float16).requires_grad_()
+                           for _ in range(3)]
+                lens = None
+                if lens_mode == "random":
+                    lens = torch.randint(1, T + 1, (B,), generator=g, device=dev, dtype=torch.int32)
+                out = streaming_attention(q, k, v, lens, context_size=16, back_contexts=2, autotune=False)
+                out.backward(torch.randn(out.shape, generator=g, device=dev, dtype=out.dtype))
+                assert torch._dynamo.utils.counters["stats"]["unique_graphs"] <= 4
     torch.cuda.synchronize()
+    assert torch.isfinite(q.grad).all()
 
 
-def test_inside_a_compiled_function(monkeypatch):
+def test_call_path_selection(monkeypatch):
+    """Direct op call by default; the compiled wrapper per call site, or process-wide through either
+    environment variable; all paths give the same bits."""
+    from streaming_attention import api, compiled_wrapper, streaming_attention
+
+    for var in ("STREAMING_ATTENTION_COMPILED", "STREAMING_ATTENTION_EAGER"):
+        monkeypatch.delenv(var, raising=False)
+    assert not api._use_compiled_wrapper()
+    with compiled_wrapper():
+        assert api._use_compiled_wrapper()
+        with compiled_wrapper(False):
+            assert not api._use_compiled_wrapper()
+        assert api._use_compiled_wrapper()
+    assert not api._use_compiled_wrapper()
+    monkeypatch.setenv("STREAMING_ATTENTION_EAGER", "1")
+    assert not api._use_compiled_wrapper()
+    monkeypatch.setenv("STREAMING_ATTENTION_EAGER", "0")
+    assert api._use_compiled_wrapper()
+    monkeypatch.delenv("STREAMING_ATTENTION_EAGER")
     monkeypatch.setenv("STREAMING_ATTENTION_COMPILED", "1")
+    assert api._use_compiled_wrapper()
+    with compiled_wrapper(False):
+        assert not api._use_compiled_wrapper()
+    monkeypatch.delenv("STREAMING_ATTENTION_COMPILED")
+    dev = torch.device("cuda:0")
+    q, k, v, _ = (t.to(dev) for t in make_inputs(2, 2, 70, 64, seed=33))
+    direct = streaming_attention(q, k, v, None, 16, 1)
+    with compiled_wrapper():
+        wrapped = streaming_attention(q, k, v, None, 16, 1)
+    assert torch.equal(direct, wrapped)
+
+
+def test_double_backward_raises():
+    """The reference registers no autograd formula for its backward op (kernel.py:1360-1442), so
+    differentiating through the backward pass raises there; here too, instead of detaching silently."""
+    from streaming_attention import streaming_attention
+
+    dev = torch.device("cuda:0")
+    q, k, v, d_o = (t.to(dev).requires_grad_() for t in make_inputs(1, 2, 40, 64, seed=34))
+    out = streaming_attention(q, k, v, None, 8, 1)
+    (dq,) = torch.autograd.grad(out, q, d_o, create_graph=True)
+    with pytest.raises(RuntimeError, match="double backward"):
+        dq.sum().backward()
+    # the ordinary backward is unaffected
+    out = streaming_attention(q, k, v, None, 8, 1)
+    out.backward(d_o.detach())
+    assert torch.isfinite(q.grad).all()
+
+
+def test_inside_a_compiled_function():
     from oracle import sa_oracle
     from streaming_attention import streaming_attention
     from tests.helpers import assert_close
