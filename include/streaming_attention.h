@@ -23,11 +23,21 @@
  *     the caller need not clear them first.  Input positions t >= lens[b] are never
  *     read, so they may hold anything.
  *   - Return value: 0 on success, > 0 a hipError_t from the launch, < 0 one of SA_ERR_*.
- *   - Re-entrant.  The library's mutable state is the per-device, per-kernel attribute set-up
+ *   - Re-entrant.  The library's mutable state is (1) the per-device, per-kernel attribute set-up
  *     (hipFuncSetAttribute on the first call of each kernel shape on each device, guarded by a
- *     mutex) and the variants pinned through sa_tune_override() (atomics; a measurement and test
- *     hook that no product caller needs).  Because of the former, the first call of each kernel
- *     shape on a device must be made outside a HIP graph capture.
+ *     mutex), (2) the variants pinned through sa_tune_override() (atomics; a measurement and test
+ *     hook that no product caller needs) and (3) the tile counters of the hand-scheduled kernels
+ *     at D = 128, described next.  Because of (1), the first call of each kernel shape on a device
+ *     must be made outside a HIP graph capture.
+ *   - Tile counters.  On a problem with at least two tiles per compute unit the hand-scheduled
+ *     forward kernel launches one workgroup per compute unit, and the workgroups take their tiles from
+ *     counters in a static device array (36 KiB per GPU, 64 blocks of counters).  A block of counters
+ *     belongs to one (device, stream) pair from that stream's first such launch to the end of the
+ *     process; launches on one stream run in order and share it, and every launch leaves it zeroed.
+ *     The pairing is kept in a small host table under a mutex.  A launch runs one workgroup per tile
+ *     instead, with identical results, when its stream is being captured into a graph (a replay may
+ *     overlap anything), when it is the per-thread default stream (one handle for many streams) and
+ *     when all 64 blocks of the device belong to other streams.  Nothing for the caller to manage.
  *   - The 16-bit dK/dV kernels at D >= 64 multiply K by -sm_scale*log2(e) and round the product to the
  *     element type before the score MFMA (what the reference does for prescale_qk=True,
  *     src/streaming_attention/kernel.py:1065-1066), whatever `prescale_qk` the caller of the Python
@@ -178,9 +188,9 @@ int sa_launch_choice(int D, int context_size, int back_contexts, int kernel);
  * variant = -1.  Meant for measurements (it is how the table was produced) and for tests that
  * exercise every variant; the counterpart of the reference's `autotune` switch
  * (src/streaming_attention/kernel.py:1154-1193).  A pinned software-pipelined variant applies to D = 128 only.
- * A measurement and test hook, not part of the operator: the pinned variants are the library's only
- * mutable state besides the per-device kernel attributes.  They are atomics, so a launch on another
- * thread sees either the old or the new variant, but which one is not ordered.  Returns 0 or SA_ERR_ARG. */
+ * A measurement and test hook, not part of the operator.  The pinned variants are atomics, so a launch
+ * on another thread sees either the old or the new variant, but which one is not ordered.  Returns 0 or
+ * SA_ERR_ARG. */
 int sa_tune_override(int kernel, int variant);
 
 /* Human-readable text for a return code of the functions above (static storage). */

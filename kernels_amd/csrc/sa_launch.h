@@ -66,9 +66,8 @@ constexpr int window_class(int chunk, int back) {
   return w < 256 ? 0 : w < 1024 ? 1 : w < 4096 ? 2 : 3;
 }
 #include "sa_tune_table.inc"
-// Variants pinned through sa_tune_override() for measurements and tests; -1 = use the table.  The only
-// mutable state of the library besides the per-device kernel attributes: atomics, so that a launch on
-// one thread reads a whole value while another thread pins or releases a variant.
+// Variants pinned through sa_tune_override() for measurements and tests; -1 = use the table.  Atomics, so
+// that a launch on one thread reads a whole value while another thread pins or releases a variant.
 extern std::atomic<int> g_tune_override[3];
 // The hand-scheduled kernels are single assembly statements over fixed registers.  A build with
 // -DSA_NO_ASM_KERNELS leaves them out (for a compiler that cannot satisfy their register constraints)
@@ -94,6 +93,18 @@ inline LaunchChoice launch_choice(int D, int chunk, int back) {
   if (!pipelined && c.fwd == FWD_PIPELINED) c.fwd = FWD_NARROW;
   return c;
 }
+
+// Counter block for a launch whose workgroups stay resident and take their tiles at run time (TileFeed in
+// sa_common.h), and the number of workgroups to launch.  `counters` is null when the launch has to run one
+// workgroup per tile instead: a stream that is being captured into a graph (a replay may overlap anything),
+// the per-thread default stream (one handle, many streams), more streams than there are blocks, or too few
+// tiles for residency to pay.  A block belongs to one (device, stream) pair for the life of the process:
+// launches on one stream run one after the other, so they can share it, and each leaves it zeroed.
+struct TileQueue {
+  uint32_t* counters;
+  int workgroups;
+};
+int tile_queue(hipStream_t stream, int64_t tiles, TileQueue& out);   // 0 or an error code; in sa_api.hip
 
 template <typename T> struct Cfg {
   static constexpr int NW = 4;                                   // waves per workgroup

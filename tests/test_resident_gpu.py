@@ -1,0 +1,115 @@
+"""The forward kernel with resident workgroups (tiles handed out at run time from per-stream counters)
+against the same kernel with one workgroup per tile.
+
+A launch is resident when its stream is not being captured, it has at least two tiles per compute unit and
+its stream owns (or can still get) a counter block; inside a graph capture the same problem runs one workgroup
+per tile.  A tile's arithmetic does not depend on which workgroup runs it or when, so the two must agree bit for
+bit: that is the check here, on top of the tolerance check against the compiler-scheduled kernel.  Launches
+that follow each other on one stream share a counter block and launches on two streams use two, both covered."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+D = 128
+
+
+def _problem(B, H, T, seed, dtype, lens_list):
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(seed)
+    q, k, v = ((torch.randn(B, H, T, D, generator=g, device=dev) * 0.5).to(dtype) for _ in range(3))
+    lens = torch.tensor(lens_list, dtype=torch.int32, device=dev) if lens_list is not None else None
+    return q, k, v, lens
+
+
+def _forward(q, k, v, lens, C, R):
+    from streaming_attention import streaming_attention
+
+    return streaming_attention(q, k, v, lens, C, R, return_lse=True)
+
+
+@pytest.fixture()
+def pipelined_forward():
+    from streaming_attention import _lib
+
+    lib = _lib.load()
+    if lib.sa_query(7) != 1:
+        pytest.skip("library built without the hand-scheduled kernels")
+    assert lib.sa_tune_override(0, 1) == 0
+    yield lib
+    lib.sa_tune_override(0, -1)
+
+
+def _enough_tiles(B, H, T):
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    return B * H * ((T + 255) // 256) >= 2 * units
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+def test_resident_forward_is_bitwise_the_per_tile_forward(pipelined_forward, dtype):
+    lib = pipelined_forward
+    B, H, T, C, R = 5, 8, 4700, 256, 8
+    assert _enough_tiles(B, H, T)
+    q, k, v, lens = _problem(B, H, T, 7, dtype, [4700, 0, 3111, 5000, 256])
+    # resident, three launches in a row on one stream (each must leave the counters ready for the next)
+    eager = [_forward(q, k, v, lens, C, R) for _ in range(3)]
+    torch.cuda.synchronize()
+    # captured: one workgroup per tile; replayed twice with eager work in between
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _forward(q, k, v, lens, C, R)          # first call of the shape outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o_g, lse_g = _forward(q, k, v, lens, C, R)
+    for _ in range(2):
+        o_g.fill_(float("nan"))
+        graph.replay()
+        between = _forward(q, k, v, lens, C, R)
+        torch.cuda.synchronize()
+        for o, lse in eager + [between]:
+            assert torch.equal(o, o_g) and torch.equal(lse, lse_g)
+    # and the compiler-scheduled kernel, to the 16-bit bar
+    lib.sa_tune_override(0, 0)
+    o_n, lse_n = _forward(q, k, v, lens, C, R)
+    lib.sa_tune_override(0, 1)
+    assert (o_n.float() - o_g.float()).abs().max().item() <= 2e-2
+    assert (lse_n - lse_g).abs().max().item() <= 1e-4
+    assert o_g[1].abs().max().item() == 0.0 and lse_g[1].abs().max().item() == 0.0      # the empty sequence
+
+
+def test_resident_forward_on_two_streams(pipelined_forward):
+    p1 = _problem(4, 8, 4608, 11, torch.bfloat16, [4608, 4000, 2222, 4608]) + (256, 8)
+    p2 = _problem(2, 16, 5000, 12, torch.bfloat16, None) + (512, 4)
+    assert _enough_tiles(4, 8, 4608) and _enough_tiles(2, 16, 5000)
+    want1, want2 = _forward(*p1), _forward(*p2)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    got1, got2 = [], []
+    for _ in range(8):          # nothing waits between the launches: the two streams overlap
+        with torch.cuda.stream(s1):
+            got1.append(_forward(*p1))
+        with torch.cuda.stream(s2):
+            got2.append(_forward(*p2))
+    torch.cuda.synchronize()
+    for o, lse in got1:
+        assert torch.equal(o, want1[0]) and torch.equal(lse, want1[1])
+    for o, lse in got2:
+        assert torch.equal(o, want2[0]) and torch.equal(lse, want2[1])
+
+
+def test_more_streams_than_counter_blocks(pipelined_forward):
+    """Streams beyond the library's counter blocks run one workgroup per tile: same results."""
+    p = _problem(4, 8, 4608, 13, torch.float16, [4608, 100, 4608, 3000]) + (256, 8)
+    want = _forward(*p)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(70)]
+    outs = []
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            outs.append(_forward(*p))
+    torch.cuda.synchronize()
+    for o, lse in outs:
+        assert torch.equal(o, want[0]) and torch.equal(lse, want[1])
