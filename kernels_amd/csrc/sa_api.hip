@@ -130,6 +130,7 @@ int sa_forward(const void* q, const void* k, const void* v, const int32_t* lens,
   p.v_sb = vs[0]; p.v_sh = vs[1]; p.v_st = vs[2];
   p.B = B; p.H = H; p.T = T; p.C = context_size; p.R = back_contexts;
   clamp_window(T, p.C, p.R);
+  p.cdiv = chunk_div(p.C > 0 ? p.C : 1);
   p.scale_log2e = sm_scale * kLog2e;
   return by_dtype(dtype, [&](auto tag) {
     using E = decltype(tag);
@@ -173,6 +174,7 @@ static int fill_bwd(BwdParams& p, const void* q, const void* k, const void* v, c
   p.do_sb = gs[0]; p.do_sh = gs[1]; p.do_st = gs[2];
   p.B = B; p.H = H; p.T = T; p.C = context_size; p.R = back_contexts;
   clamp_window(T, p.C, p.R);
+  p.cdiv = chunk_div(p.C > 0 ? p.C : 1);
   p.scale = sm_scale;
   p.scale_log2e = sm_scale * kLog2e;
   return SA_OK;

@@ -67,6 +67,7 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(const BwdParams p) {
   tile_coords(blockIdx.x, gridDim.x, p.n_tiles, bh, qt);
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
+  auto cdiv = [&](int x) { return div_by(x, p.cdiv); };   // x / C
 
   int L = T_;
   if (p.lens) {
@@ -83,16 +84,16 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(const BwdParams p) {
 
   const int qrow = q0 + wave * 32 + c;
   const int qe = qrow < L ? qrow : L - 1;
-  const int qchunk = qe / C;
+  const int qchunk = cdiv(qe);
   const int lo = (qchunk > R ? qchunk - R : 0) * C;
   const int hi = (qchunk + 1) * C < L ? (qchunk + 1) * C : L;
   const int wq_first = q0 + wave * 32 < L ? q0 + wave * 32 : L - 1;
   const int wq_last = q0 + wave * 32 + 31 < L ? q0 + wave * 32 + 31 : L - 1;
-  const int hi_min = (wq_first / C + 1) * C < L ? (wq_first / C + 1) * C : L;
-  const int lo_max = (wq_last / C > R ? wq_last / C - R : 0) * C;
+  const int hi_min = (cdiv(wq_first) + 1) * C < L ? (cdiv(wq_first) + 1) * C : L;
+  const int lo_max = (cdiv(wq_last) > R ? cdiv(wq_last) - R : 0) * C;
   const int gq_last = q0 + TQ - 1 < L ? q0 + TQ - 1 : L - 1;
-  const int lo_wg = (q0 / C > R ? q0 / C - R : 0) * C;
-  const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
+  const int lo_wg = (cdiv(q0) > R ? cdiv(q0) - R : 0) * C;
+  const int hi_wg = (cdiv(gq_last) + 1) * C < L ? (cdiv(gq_last) + 1) * C : L;
   const int kt0 = lo_wg / TK, kt1 = (hi_wg + TK - 1) / TK;
 
   const float sl2e = fabsf(p.scale_log2e);
@@ -222,6 +223,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   tile_coords(blockIdx.x, gridDim.x, p.n_tiles, bh, kt);
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
+  auto cdiv = [&](int x) { return div_by(x, p.cdiv); };   // x / C
 
   int L = T_;
   if (p.lens) {
@@ -239,9 +241,9 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(const BwdParams p) {
   }
 
   // query window [qlo, qhi) of a key: its own chunk and the R chunks after it, below L
-  auto win_lo = [&](int key) { return (key / C) * C; };
+  auto win_lo = [&](int key) { return (cdiv(key)) * C; };
   auto win_hi = [&](int key) {
-    const int64_t e = ((int64_t)(key / C) + R + 1) * (int64_t)C;
+    const int64_t e = ((int64_t)(cdiv(key)) + R + 1) * (int64_t)C;
     return e < (int64_t)L ? (int)e : L;
   };
   const int krow = k0 + wave * 32 + c;
@@ -425,6 +427,7 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
   tile_coords(blockIdx.x, gridDim.x, p.n_tiles, bh, qt, growing_tiles(p.C, p.R, p.T, NW * 32));
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
+  auto cdiv = [&](int x) { return div_by(x, p.cdiv); };   // x / C
 
   int L = T_;
   if (p.lens) {
@@ -443,20 +446,20 @@ __global__ __launch_bounds__(NW * 64) void dq2_kernel(const BwdParams p) {
 
   const int qrow = q0 + wave * 32 + c;
   const int qe = qrow < L ? qrow : L - 1;
-  const int qchunk = qe / C;
+  const int qchunk = cdiv(qe);
   const int lo = (qchunk > R ? qchunk - R : 0) * C;
   const int hi = (qchunk + 1) * C < L ? (qchunk + 1) * C : L;
   const int wq_first = q0 + wave * 32 < L ? q0 + wave * 32 : L - 1;
   const int wq_last = q0 + wave * 32 + 31 < L ? q0 + wave * 32 + 31 : L - 1;
-  const int hi_min = (wq_first / C + 1) * C < L ? (wq_first / C + 1) * C : L;
-  const int lo_max = (wq_last / C > R ? wq_last / C - R : 0) * C;
+  const int hi_min = (cdiv(wq_first) + 1) * C < L ? (cdiv(wq_first) + 1) * C : L;
+  const int lo_max = (cdiv(wq_last) > R ? cdiv(wq_last) - R : 0) * C;
   // keys any query of this wave can see; a wave whose queries are all padding sees none
   const bool wave_live = q0 + wave * 32 < L;
-  const int lo_min = (wq_first / C > R ? wq_first / C - R : 0) * C;
-  const int hi_max = !wave_live ? 0 : ((wq_last / C + 1) * C < L ? (wq_last / C + 1) * C : L);
+  const int lo_min = (cdiv(wq_first) > R ? cdiv(wq_first) - R : 0) * C;
+  const int hi_max = !wave_live ? 0 : ((cdiv(wq_last) + 1) * C < L ? (cdiv(wq_last) + 1) * C : L);
   const int gq_last = q0 + TQ - 1 < L ? q0 + TQ - 1 : L - 1;
-  const int lo_wg = (q0 / C > R ? q0 / C - R : 0) * C;
-  const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
+  const int lo_wg = (cdiv(q0) > R ? cdiv(q0) - R : 0) * C;
+  const int hi_wg = (cdiv(gq_last) + 1) * C < L ? (cdiv(gq_last) + 1) * C : L;
   const int kt0 = lo_wg / TK, kt1 = (hi_wg + TK - 1) / TK;
 
   const float sl2e = fabsf(p.scale_log2e);
@@ -610,6 +613,7 @@ __global__ __launch_bounds__(NW * 64, (D == 64 ? 3 : 1)) void dkdv2_kernel(const
                   p.lens_stride, bh, kt, L);
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
+  auto cdiv = [&](int x) { return div_by(x, p.cdiv); };   // x / C
   const int k0 = kt * TKB;
   T* dk_base = reinterpret_cast<T*>(p.dk) + (int64_t)bh * T_ * D;
   T* dv_base = reinterpret_cast<T*>(p.dv) + (int64_t)bh * T_ * D;
@@ -620,9 +624,9 @@ __global__ __launch_bounds__(NW * 64, (D == 64 ? 3 : 1)) void dkdv2_kernel(const
     return;
   }
 
-  auto win_lo = [&](int key) { return (key / C) * C; };
+  auto win_lo = [&](int key) { return (cdiv(key)) * C; };
   auto win_hi = [&](int key) {
-    const int64_t e = ((int64_t)(key / C) + R + 1) * (int64_t)C;
+    const int64_t e = ((int64_t)(cdiv(key)) + R + 1) * (int64_t)C;
     return e < (int64_t)L ? (int)e : L;
   };
   const int krow = k0 + wave * 32 + c;

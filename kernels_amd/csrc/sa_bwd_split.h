@@ -61,6 +61,7 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
                   p.lens_stride, bh, kt, L);
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
+  auto cdiv = [&](int x) { return div_by(x, p.cdiv); };   // x / C
   const int k0 = kt * TKB;
   T* dk_base = reinterpret_cast<T*>(p.dk) + (int64_t)bh * T_ * D;
   T* dv_base = reinterpret_cast<T*>(p.dv) + (int64_t)bh * T_ * D;
@@ -71,9 +72,9 @@ __global__ __launch_bounds__(512) void dkdv_split_kernel(const BwdParams p) {
     return;
   }
 
-  auto win_lo = [&](int key) { return (key / C) * C; };
+  auto win_lo = [&](int key) { return (cdiv(key)) * C; };
   auto win_hi = [&](int key) {
-    const int64_t e = ((int64_t)(key / C) + R + 1) * (int64_t)C;
+    const int64_t e = ((int64_t)(cdiv(key)) + R + 1) * (int64_t)C;
     return e < (int64_t)L ? (int)e : L;
   };
   const int krow = k0 + pair * 32 + c;

@@ -525,6 +525,16 @@ template <int N> SA_DEV void wait_loads() {
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
+// Waits until at most min(ahead, MAXA) tiles of LPT loads each are outstanding (ahead is wave-uniform).
+template <int LPT, int MAXA> SA_DEV void wait_tiles(int ahead) {
+  if constexpr (MAXA <= 0) {
+    wait_loads<0>();
+  } else {
+    if (ahead >= MAXA) wait_loads<MAXA * LPT>();
+    else wait_tiles<LPT, MAXA - 1>(ahead);
+  }
+}
+
 // Cooperative copy of a [ROWS][D] row-major global tile into registers and on into an
 // LDS tile.  Rows are clamped to `last_row` so that a ragged final tile reads valid
 // memory (the values are masked by the caller).
@@ -804,6 +814,27 @@ SA_DEV void store_rows_coalesced(T* patch, T* out_rows, int rows_valid, const f3
   }
 }
 
+// Division of a position below 2^31 by the chunk size without the hardware's 30-instruction emulation:
+// with l = ceil(log2(d)) and m = ceil(2^(31+l) / d) (m < 2^32), n / d == (n * m) >> (31 + l) for every
+// 0 <= n < 2^31 (Granlund and Montgomery, "Division by invariant integers using multiplication", 1994).
+struct ChunkDiv {
+  uint32_t mul, shift;
+};
+constexpr ChunkDiv chunk_div(int d) {   // d >= 1
+  uint32_t l = 0;
+  while ((1ull << l) < (unsigned long long)d) ++l;
+  const unsigned long long two = 1ull << (31 + l);
+  return ChunkDiv{(uint32_t)((two + (unsigned long long)d - 1) / (unsigned long long)d), 31 + l};
+}
+constexpr int div_by(int n, ChunkDiv c) { return (int)(((unsigned long long)(uint32_t)n * c.mul) >> c.shift); }
+static_assert(div_by(0x7fffffff, chunk_div(1)) == 0x7fffffff && div_by(12345, chunk_div(1)) == 12345, "d = 1");
+static_assert(div_by(0x7fffffff, chunk_div(2)) == 0x3fffffff && div_by(0x7ffffffe, chunk_div(0x7fffffff)) == 0 &&
+              div_by(0x7fffffff, chunk_div(0x7fffffff)) == 1, "extremes");
+static_assert(div_by(2999, chunk_div(10)) == 299 && div_by(3000, chunk_div(10)) == 300 && div_by(95, chunk_div(96)) == 0 &&
+              div_by(96, chunk_div(96)) == 1 && div_by(0x7fffffff, chunk_div(10)) == 214748364 &&
+              div_by(0x7fffffff, chunk_div(3)) == 715827882 && div_by(0x7fffffff, chunk_div(641)) == 3350208 &&
+              div_by(65535, chunk_div(256)) == 255 && div_by(0x7fffffff, chunk_div(10000)) == 214748, "samples");
+
 struct FwdParams {
   const void *q, *k, *v;
   void* o;          // contiguous [B,H,T,D]
@@ -816,6 +847,7 @@ struct FwdParams {
   int n_tiles;        // query tiles per (b,h)
   int n_blocks;       // B * H * n_tiles
   uint32_t* feed;     // counter block of a launch with resident workgroups (TileFeed), or null
+  ChunkDiv cdiv;      // division by C
 };
 
 struct BwdParams {
@@ -833,6 +865,7 @@ struct BwdParams {
   const void* o;
   int64_t o_sb, o_sh, o_st;
   float* delta_out;
+  ChunkDiv cdiv;      // division by C
 };
 
 struct DeltaParams {

@@ -32,6 +32,7 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
   tile_coords(blockIdx.x, gridDim.x, p.n_tiles, bh, qt);
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
+  auto cdiv = [&](int x) { return div_by(x, p.cdiv); };   // x / C
 
   int L = T_;
   if (p.lens) {
@@ -53,18 +54,18 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(const FwdParams p) {
   // ---- per-lane query and its key window ------------------------------------------
   const int qrow = q0 + wave * 32 + c;
   const int qe = qrow < L ? qrow : L - 1;  // rows past L mimic the last valid row
-  const int qchunk = qe / C;
+  const int qchunk = cdiv(qe);
   const int lo = (qchunk > R ? qchunk - R : 0) * C;
   const int hi = (qchunk + 1) * C < L ? (qchunk + 1) * C : L;
   // the tightest window over the wave decides whether a tile needs masking at all
   const int wq_first = q0 + wave * 32 < L ? q0 + wave * 32 : L - 1;
   const int wq_last = q0 + wave * 32 + 31 < L ? q0 + wave * 32 + 31 : L - 1;
-  const int hi_min = (wq_first / C + 1) * C < L ? (wq_first / C + 1) * C : L;
-  const int lo_max = (wq_last / C > R ? wq_last / C - R : 0) * C;
+  const int hi_min = (cdiv(wq_first) + 1) * C < L ? (cdiv(wq_first) + 1) * C : L;
+  const int lo_max = (cdiv(wq_last) > R ? cdiv(wq_last) - R : 0) * C;
   // union over the workgroup decides which tiles are visited
   const int gq_last = q0 + TQ - 1 < L ? q0 + TQ - 1 : L - 1;
-  const int lo_wg = (q0 / C > R ? q0 / C - R : 0) * C;
-  const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
+  const int lo_wg = (cdiv(q0) > R ? cdiv(q0) - R : 0) * C;
+  const int hi_wg = (cdiv(gq_last) + 1) * C < L ? (cdiv(gq_last) + 1) * C : L;
   const int kt0 = lo_wg / TK, kt1 = (hi_wg + TK - 1) / TK;
 
   const float sl2e = fabsf(p.scale_log2e);
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   using E = Elem<T>;
   using G = TileGeom<T, D>;
   using Frag = typename E::Frag;
-  static_assert(G::SWZ && (NST == 2 || NST == 3), "swizzled 16-bit tiles, 2 or 3 stages");
+  static_assert(G::SWZ && NST >= 2 && (NST - 2) * 2 * AsyncTile<T, D, TK, NW>::PER_WAVE < 64, "swizzled 16-bit tiles; the loads of NST-2 tiles fit the load counter");
   constexpr int WQ = QB * 32, TQ = NW * WQ, NT = NW * 64, KBN = TK / 32;
   constexpr int NF = G::NF, DB = G::DB;
   constexpr int TILE = TK * D;            // elements per K or V tile
@@ -245,6 +246,7 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   tile_coords(blockIdx.x, gridDim.x, p.n_tiles, bh, qt, SHORT ? growing_tiles(p.C, p.R, p.T, NW * QB * 32) : 0);
   const int hd = bh % p.H, b = bh / p.H;
   const int T_ = p.T, C = p.C, R = p.R;
+  auto cdiv = [&](int x) { return div_by(x, p.cdiv); };   // x / C
 
   int L = T_;
   if (p.lens) {
@@ -268,21 +270,21 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   for (int qb = 0; qb < QB; ++qb) {
     qrow[qb] = q0 + wave * WQ + qb * 32 + c;
     const int qe = qrow[qb] < L ? qrow[qb] : L - 1;
-    const int qchunk = qe / C;
+    const int qchunk = cdiv(qe);
     lo[qb] = (qchunk > R ? qchunk - R : 0) * C;
     hi[qb] = (qchunk + 1) * C < L ? (qchunk + 1) * C : L;
   }
   const int wq_first = q0 + wave * WQ < L ? q0 + wave * WQ : L - 1;
   const int wq_last = q0 + wave * WQ + WQ - 1 < L ? q0 + wave * WQ + WQ - 1 : L - 1;
-  const int hi_min = (wq_first / C + 1) * C < L ? (wq_first / C + 1) * C : L;
-  const int lo_max = (wq_last / C > R ? wq_last / C - R : 0) * C;
+  const int hi_min = (cdiv(wq_first) + 1) * C < L ? (cdiv(wq_first) + 1) * C : L;
+  const int lo_max = (cdiv(wq_last) > R ? cdiv(wq_last) - R : 0) * C;
   // keys any query of this wave can see; a wave whose queries are all padding sees none
   const bool wave_live = q0 + wave * WQ < L;
-  const int lo_min = (wq_first / C > R ? wq_first / C - R : 0) * C;
-  const int hi_max = !wave_live ? 0 : ((wq_last / C + 1) * C < L ? (wq_last / C + 1) * C : L);
+  const int lo_min = (cdiv(wq_first) > R ? cdiv(wq_first) - R : 0) * C;
+  const int hi_max = !wave_live ? 0 : ((cdiv(wq_last) + 1) * C < L ? (cdiv(wq_last) + 1) * C : L);
   const int gq_last = q0 + TQ - 1 < L ? q0 + TQ - 1 : L - 1;
-  const int lo_wg = (q0 / C > R ? q0 / C - R : 0) * C;
-  const int hi_wg = (gq_last / C + 1) * C < L ? (gq_last / C + 1) * C : L;
+  const int lo_wg = (cdiv(q0) > R ? cdiv(q0) - R : 0) * C;
+  const int hi_wg = (cdiv(gq_last) + 1) * C < L ? (cdiv(gq_last) + 1) * C : L;
   const int kt0 = lo_wg / TK, kt1 = (hi_wg + TK - 1) / TK;
 
   // never exactly 0, so that a masked score of -inf stays -inf after scaling
@@ -333,9 +335,9 @@ __global__ __launch_bounds__(NW * 64) void fwd2_kernel(const FwdParams p) {
   wait_all_loads();   // Q fragments (and, as loads complete in order, the first tiles)
 
   for (int t = kt0; t < kt1; ++t) {
-    // tile t has landed once at most the younger tiles' loads are outstanding
-    if (NST == 3 && t + 1 < kt1) wait_loads<LPT>();
-    else wait_loads<0>();
+    // tile t has landed once at most the loads of the younger tiles are outstanding: NST-2 of them, fewer
+    // near the end of the window
+    wait_tiles<LPT, NST - 2>(kt1 - 1 - t);
     __syncthreads();   // every wave's share is visible; stage (t-1) % NST is free again
     if (t + NST - 1 < kt1) issue_tile(t + NST - 1);
 
