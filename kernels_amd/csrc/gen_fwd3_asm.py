@@ -38,12 +38,13 @@ Register map (D = 128):
   v187, v188 block maximum      v189, v190 block sums    v[191:198] exp2 temporaries    v[199:207] temporaries
   v[208:239] wave-uniform inputs, copied to s40... at entry (see SCALARS)
   v240, v241 buffer offsets of this lane for the K / V tile loads
-  s40 |scale*log2e|  s41 one past the last key tile  s42 key tile of even block j  s43 first key of block j
+  s40 |scale*log2e|  s41 one past the last key tile of the workgroup  s42 key tile of even block j  s43 first key of block j
   s44..s47 LDS address of the stages of tiles s42-1, s42, s42+1, s42+2  s48 wave offset inside a tile for the
   asynchronous loads  s49 -inf  s50, s51: a block inside [s50, s51) lies inside the window of every query of
   this wave  s[52:55], s[56:59] buffer resources of K and V  s60, s61 their running byte offsets  s62, s63 bytes
   between a wave's load instructions  s64, s65 bytes between tiles  s66..s69 temporaries  s[70:75] lane masks
   s76 set when the accumulators must be rescaled at the end of the iteration
+  s77, s78 first key tile of this wave's own window and one past its last
 
 Run:  python3 gen_fwd3_asm.py > sa_fwd3_asm.inc   (the Makefile does this)
 """
@@ -366,7 +367,9 @@ class Gen:
 
 SCALARS = ["sl2e", "kt1", "t", "kb", "st0", "st1", "st2", "st3", "wave_tile", "ninf", "lo_max", "hi_min",
            "rk0", "rk1", "rk2", "rk3", "rv0", "rv1", "rv2", "rv3", "soff_k", "soff_v", "istep_k", "istep_v",
-           "tstep_k", "tstep_v"]          # v208 + i  ->  s40 + i
+           "tstep_k", "tstep_v", "wfirst", "wend"]   # v208 + i -> s40 + i; the last two -> s77, s78 (s66..s76 are taken)
+SREG = {i: 40 + i for i in range(26)}
+SREG.update({26: 77, 27: 78})
 
 
 def issue_tile():
@@ -389,8 +392,30 @@ def issue_tile():
 def generate(dt):
     L = lambda name: f"{name}_{dt}_%="
     g = Gen(dt)
+    # tile hand-over of an even iteration: tile s42 + 1 must have landed in every wave's share before its K
+    # is read (slot 18 on); the stage of tile s42 - 2 (s47), which nobody reads any more, takes tile s42 + 2
+    def mid(lab):
+        return ["s_add_i32 s66, s42, 1",
+                "s_cmp_ge_i32 s66, s41",
+                f"s_cbranch_scc1 Lskip_{lab}",
+                "s_waitcnt vmcnt(0)",
+                "s_barrier",
+                "s_add_i32 s66, s42, 2",
+                "s_cmp_ge_i32 s66, s41",
+                f"s_cbranch_scc1 Lskip_{lab}"] + issue_tile() + [f"Lskip_{lab}:"]
+    rotate = ["s_mov_b32 s66, s44", "s_mov_b32 s44, s45", "s_mov_b32 s45, s46", "s_mov_b32 s46, s47", "s_mov_b32 s47, s66"]
     # ---- prologue: scalars, per-lane state, addresses, scores of block 0, ring entries of the first iteration
-    pro = [f"v_readfirstlane_b32 s{40 + i}, v{208 + i}" for i in range(len(SCALARS))]
+    pro = [f"v_readfirstlane_b32 s{SREG[i]}, v{208 + i}" for i in range(len(SCALARS))]
+    # Tiles of the workgroup's window that lie before this wave's own window (s77 = its first tile): no arithmetic,
+    # only the wave's part in the hand-over of every tile (its share of the loads, the barrier).  The same after
+    # the wave's last tile (s78 = one past it).
+    pro += [L("Lin") + ":",
+            "s_cmp_ge_i32 s42, s77",
+            "s_cbranch_scc1 " + L("Lin_done")] + mid(L("i")) + [
+            "s_add_i32 s42, s42, 1"] + rotate + [
+            "s_branch " + L("Lin"),
+            L("Lin_done") + ":",
+            "s_lshl_b32 s43, s42, 6"]
     pro += ["s_mov_b32 s76, 0"]
     for qb in range(2):
         pro += [f"v_mov_b32 {vr(M + qb)}, s49", f"v_mov_b32 {vr(LRUN + qb)}, 0",
@@ -413,17 +438,6 @@ def generate(dt):
         g.fetch(NFRAG + f, f, 0)
     text = g.out
 
-    # tile hand-over of an even iteration: tile s42 + 1 must have landed in every wave's share before its K
-    # is read (slot 18 on); the stage of tile s42 - 2 (s47), which nobody reads any more, takes tile s42 + 2
-    def mid(lab):
-        return ["s_add_i32 s66, s42, 1",
-                "s_cmp_ge_i32 s66, s41",
-                f"s_cbranch_scc1 Lskip_{lab}",
-                "s_waitcnt vmcnt(0)",
-                "s_barrier",
-                "s_add_i32 s66, s42, 2",
-                "s_cmp_ge_i32 s66, s41",
-                f"s_cbranch_scc1 Lskip_{lab}"] + issue_tile() + [f"Lskip_{lab}:"]
     k = 1
     first = g.body(k, 0, L("f"), with_pv=False, mid=mid(L("f")))
     k += 1
@@ -440,8 +454,8 @@ def generate(dt):
     text += b1
     text += ["s_add_i32 s42, s42, 1",
              "s_add_i32 s43, s43, 32",
-             "s_mov_b32 s66, s44", "s_mov_b32 s44, s45", "s_mov_b32 s45, s46", "s_mov_b32 s46, s47", "s_mov_b32 s47, s66",
-             "s_cmp_ge_i32 s42, s41",
+             *rotate,
+             "s_cmp_ge_i32 s42, s78",
              "s_cbranch_scc1 " + L("Lend")]
     text += b0
     text += ["s_branch " + L("Lloop"),
@@ -459,8 +473,13 @@ def generate(dt):
         text.append(f"s_waitcnt lgkmcnt({min(n, 15)})")
         for qb in range(2):
             text.append(f"{g.mfma} {O(qb, m)}, {RG(x)}, {PB(1, qb, half)}, {O(qb, m)}")
-    text += ["s_nop 15", "s_nop 15", "s_nop 15", "s_nop 15",
-             "s_branch " + L("Lout")]
+    text += ["s_nop 15", "s_nop 15", "s_nop 15", "s_nop 15"]
+    # tiles of the workgroup's window after this wave's last one
+    text += [L("Lfin") + ":",
+             "s_cmp_ge_i32 s42, s41",
+             "s_cbranch_scc1 " + L("Lout")] + mid(L("x")) + [
+             "s_add_i32 s42, s42, 1"] + rotate + [
+             "s_branch " + L("Lfin")]
     text += g.tails
     text.append(L("Lout") + ":")
     name = f"SA_FWD3_128_{dt.upper()}"
