@@ -44,6 +44,9 @@ WORKLOADS = {
     "headline_bf16_T16384_D128": (4, 16, 16384, 128, "bfloat16", 256, 8, "uniform_half_full", 1.0),
     "ragged_fp16_T2048_D128": (16, 8, 2048, 128, "float16", 64, 1, "loguniform_64_T", 1.0),
     "long_bf16_T65536_D128": (1, 32, 65536, 128, "bfloat16", 512, 16, "full", 1.0),
+    # the largest shapes of the reference's own benchmark grid (benchmark/benchmark_streaming_attention.py:43-111), for profiling
+    "refgrid_fp16_T3000_D64_C10": (128, 12, 3000, 64, "float16", 10, 9, "full", 1.0),
+    "refgrid_fp16_T3000_D64_C32": (128, 12, 3000, 64, "float16", 32, 2, "full", 1.0),
 }
 DEFAULT = "headline_bf16_T16384_D128"
 
