@@ -23,21 +23,11 @@
  *     the caller need not clear them first.  Input positions t >= lens[b] are never
  *     read, so they may hold anything.
  *   - Return value: 0 on success, > 0 a hipError_t from the launch, < 0 one of SA_ERR_*.
- *   - Re-entrant.  The library's mutable state is (1) the per-device, per-kernel attribute set-up
+ *   - Re-entrant.  The library's mutable state is the per-device, per-kernel attribute set-up
  *     (hipFuncSetAttribute on the first call of each kernel shape on each device, guarded by a
- *     mutex), (2) the variants pinned through sa_tune_override() (atomics; a measurement and test
- *     hook that no product caller needs) and (3) the tile counters of the hand-scheduled kernels
- *     at D = 128, described next.  Because of (1), the first call of each kernel shape on a device
- *     must be made outside a HIP graph capture.
- *   - Tile counters.  On a problem with at least two tiles per compute unit the hand-scheduled
- *     forward kernel launches one workgroup per compute unit, and the workgroups take their tiles from
- *     counters in a static device array (36 KiB per GPU, 64 blocks of counters).  A block of counters
- *     belongs to one (device, stream) pair from that stream's first such launch to the end of the
- *     process; launches on one stream run in order and share it, and every launch leaves it zeroed.
- *     The pairing is kept in a small host table under a mutex.  A launch runs one workgroup per tile
- *     instead, with identical results, when its stream is being captured into a graph (a replay may
- *     overlap anything), when it is the per-thread default stream (one handle for many streams) and
- *     when all 64 blocks of the device belong to other streams.  Nothing for the caller to manage.
+ *     mutex) and the variants pinned through sa_tune_override() (atomics; a measurement and test
+ *     hook that no product caller needs).  Because of the former, the first call of each kernel
+ *     shape on a device must be made outside a HIP graph capture.
  *   - The 16-bit dK/dV kernels at D >= 64 multiply K by -sm_scale*log2(e) and round the product to the
  *     element type before the score MFMA (what the reference does for prescale_qk=True,
  *     src/streaming_attention/kernel.py:1065-1066), whatever `prescale_qk` the caller of the Python

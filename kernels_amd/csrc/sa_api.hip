@@ -11,57 +11,8 @@ using namespace sa;
 // for the symbol; the memory is reached through the address hipGetSymbolAddress returns.
 static __device__ __align__(256) float sa_static_delta[SA_STATIC_MAX_ROWS];
 
-// Counter blocks of the launches with resident workgroups, one block per stream that has launched one
-// (at most SA_FEED_STREAMS per GPU).  One copy per GPU, reached through hipGetSymbolAddress like the array
-// above; zero when the module is loaded, and every launch leaves its block zeroed.
-constexpr int SA_FEED_STREAMS = 64;
-static __device__ __align__(256) uint32_t sa_feed_counters[SA_FEED_STREAMS * sa::SA_FEED_WORDS];
-
 namespace sa {
 std::atomic<int> g_tune_override[3] = {{-1}, {-1}, {-1}};
-
-int tile_queue(hipStream_t stream, int64_t tiles, TileQueue& out) {
-  constexpr int kMaxDevices = 64;
-  struct PerDevice {
-    uint32_t* base = nullptr;
-    int units = 0;                          // compute units
-    int used = 0;
-    hipStream_t streams[SA_FEED_STREAMS] = {};
-  };
-  static std::mutex mu;
-  static PerDevice table[kMaxDevices];
-  out.counters = nullptr;
-  out.workgroups = (int)tiles;
-  if (stream == hipStreamPerThread) return 0;
-  int dev = 0;
-  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
-  if (dev < 0 || dev >= kMaxDevices) return 0;
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  if (hipError_t e = hipStreamIsCapturing(stream, &capture); e != hipSuccess) return (int)e;
-  if (capture != hipStreamCaptureStatusNone) return 0;
-  std::lock_guard<std::mutex> lock(mu);
-  PerDevice& d = table[dev];
-  if (!d.base) {
-    void* ptr = nullptr;
-    if (hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(sa_feed_counters)); e != hipSuccess) return (int)e;
-    int units = 0;
-    if (hipError_t e = hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev); e != hipSuccess)
-      return (int)e;
-    d.units = units;
-    d.base = static_cast<uint32_t*>(ptr);
-  }
-  // residency pays when a workgroup gets several tiles
-  if (d.units <= 0 || tiles < 2 * (int64_t)d.units) return 0;
-  int slot = 0;
-  while (slot < d.used && d.streams[slot] != stream) ++slot;
-  if (slot == d.used) {
-    if (d.used == SA_FEED_STREAMS) return 0;
-    d.streams[d.used++] = stream;
-  }
-  out.counters = d.base + (size_t)slot * SA_FEED_WORDS;
-  out.workgroups = d.units;
-  return 0;
-}
 }  // namespace sa
 
 namespace {

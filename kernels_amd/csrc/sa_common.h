@@ -645,103 +645,6 @@ SA_DEV void key_tile_coords(int bid, int n_blocks, int n_tiles, int n_end, int R
   }
 }
 
-// ---- tiles handed out at run time -----------------------------------------------------------------
-// A kernel whose workgroups stay resident (one per compute unit) and take tile after tile hides, behind the
-// work of one tile, what a workgroup per tile pays between tiles: the dispatch, the argument and length loads,
-// the first key and query loads, the drain of the last stores.  The tiles come from eight counters, one per
-// XCD, over the same block order that tile_coords maps (block id = 8 * position + XCD): a workgroup takes from
-// the counter of the XCD it runs on until that list is used up, then from the next XCD's list, and so on, so
-// that neighbouring tiles still meet in one L2 and the chip stays balanced to the last tile.
-//
-// Counter block (uint32_t words, each on its own 64 bytes): [16 * x] next position of XCD x, [16 * 8] number of
-// workgroups that have left.  All zero between launches: the last workgroup to leave clears the block.  The
-// block belongs to one launch at a time (the host hands one block to each stream).  Without a counter block a
-// workgroup runs the tile of its own block id and nothing else.
-constexpr int SA_FEED_STRIDE = 16;                      // words between counters
-constexpr int SA_FEED_WORDS = 9 * SA_FEED_STRIDE;       // per counter block
-struct TileFeed {
-  uint32_t* ctr;
-  int n_blocks;
-  int xcd, probe;   // own XCD; lists found used up so far
-
-  SA_DEV void init(uint32_t* counters, int blocks) {
-    ctr = counters;
-    n_blocks = blocks;
-    probe = 0;
-    uint32_t id;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(id));
-    xcd = (int)(id & 7u);
-  }
-  SA_DEV uint32_t add(int x) const {
-    return __hip_atomic_fetch_add(ctr + SA_FEED_STRIDE * x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  // thread 0 only: a block id from the lists not yet found used up, or -1
-  SA_DEV int take() {
-    while (probe < 8) {
-      const int x = (xcd + probe) & 7;
-      const int64_t bid = (int64_t)add(x) * 8 + x;
-      if (bid < n_blocks) return (int)bid;
-      ++probe;
-    }
-    return -1;
-  }
-  SA_DEV int share(int* slot, int tid, int bid) const {
-    if (tid == 0) *slot = bid;
-    __syncthreads();
-    const int r = __builtin_amdgcn_readfirstlane(*slot);
-    return r;
-  }
-  // the workgroup's first tile
-  SA_DEV int first(int* slot, int tid) {
-    if (!ctr) return (int)blockIdx.x < n_blocks ? (int)blockIdx.x : -1;
-    int bid = 0;
-    if (tid == 0) bid = take();
-    return share(slot, tid, bid);
-  }
-  // the next tile, waited for (the slot must not be in use: call share()'s barrier apart)
-  SA_DEV int next_blocking(int* slot, int tid) {
-    if (!ctr) return -1;
-    __syncthreads();   // everybody has read the slot's last value
-    int bid = 0;
-    if (tid == 0) bid = take();
-    return share(slot, tid, bid);
-  }
-  // Split form around a long piece of work: ask() starts the request, resolve() completes it (with a
-  // workgroup barrier) and returns the block id or -1.
-  SA_DEV uint32_t ask(int tid) const {
-    uint32_t t = 0;
-    if (ctr && tid == 0 && probe < 8) t = add((xcd + probe) & 7);
-    return t;
-  }
-  SA_DEV int resolve(uint32_t ticket, int* slot, int tid) {
-    // read by every lane on every path: the wait for the answer then has one place, here, instead of
-    // wherever the compiler next reuses the register on a path that skipped the read
-    const uint32_t answer = (uint32_t)__builtin_amdgcn_readfirstlane((int)ticket);
-    int bid = -1;
-    if (ctr && tid == 0 && probe < 8) {
-      const int x = (xcd + probe) & 7;
-      const int64_t b = (int64_t)answer * 8 + x;
-      if (b < n_blocks) bid = (int)b;
-      else {
-        ++probe;
-        bid = take();
-      }
-    }
-    return share(slot, tid, bid);
-  }
-  // every workgroup, once, after its last request
-  SA_DEV void finish(int tid) const {
-    if (!ctr || tid != 0) return;
-    uint32_t* done = ctr + SA_FEED_STRIDE * 8;
-    const uint32_t d = __hip_atomic_fetch_add(done, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    if (d == gridDim.x - 1) {
-      for (int x = 0; x < 8; ++x)
-        __hip_atomic_store(ctr + SA_FEED_STRIDE * x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(done, 0u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
-};
-
 // Number of leading query tiles of ROWS rows whose windows are still growing: rows below back_contexts chunks.
 SA_DEV int growing_tiles(int C, int R, int T, int ROWS) {
   const int64_t rows = (int64_t)C * (int64_t)R;
@@ -845,8 +748,6 @@ struct FwdParams {
   int B, H, T, C, R;
   float scale_log2e;  // sm_scale * log2(e); sign carried separately
   int n_tiles;        // query tiles per (b,h)
-  int n_blocks;       // B * H * n_tiles
-  uint32_t* feed;     // counter block of a launch with resident workgroups (TileFeed), or null
   ChunkDiv cdiv;      // division by C
 };
 

@@ -110,13 +110,8 @@ template <int D> static int fwd3_launch(FwdParams p, hipStream_t st) {
     if (int rc = prepare(kern, lds, once)) return rc;
     p.n_tiles = (int)ceil_div(p.T, TQ);
     const int64_t blocks = (int64_t)p.B * p.H * p.n_tiles;
-    if (blocks > 0x7fffffffLL / 8) return SA_ERR_TOO_LARGE;
-    if (blocks == 0) return 0;
-    TileQueue tq;
-    if (int rc = tile_queue(st, blocks, tq)) return rc;
-    p.n_blocks = (int)blocks;
-    p.feed = tq.counters;
-    hipLaunchKernelGGL(kern, dim3((unsigned)tq.workgroups), dim3(NW * 64), lds, st, p);
+    if (blocks > 0x7fffffffLL) return SA_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NW * 64), lds, st, p);
     return (int)hipGetLastError();
   } else {
     return SA_ERR_HEAD_DIM;

@@ -94,18 +94,6 @@ inline LaunchChoice launch_choice(int D, int chunk, int back) {
   return c;
 }
 
-// Counter block for a launch whose workgroups stay resident and take their tiles at run time (TileFeed in
-// sa_common.h), and the number of workgroups to launch.  `counters` is null when the launch has to run one
-// workgroup per tile instead: a stream that is being captured into a graph (a replay may overlap anything),
-// the per-thread default stream (one handle, many streams), more streams than there are blocks, or too few
-// tiles for residency to pay.  A block belongs to one (device, stream) pair for the life of the process:
-// launches on one stream run one after the other, so they can share it, and each leaves it zeroed.
-struct TileQueue {
-  uint32_t* counters;
-  int workgroups;
-};
-int tile_queue(hipStream_t stream, int64_t tiles, TileQueue& out);   // 0 or an error code; in sa_api.hip
-
 template <typename T> struct Cfg {
   static constexpr int NW = 4;                                   // waves per workgroup
   // 16-bit, D in {64, 128, 256}: forward kernel with QB query blocks per wave and NST LDS stages.
