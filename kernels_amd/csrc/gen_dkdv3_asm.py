@@ -85,8 +85,6 @@ class Gen:
     def RG(self, r, lo=0, n=4):
         # the second half of the ring lives in accumulation registers: LDS reads can land there and MFMAs can
         # take their A operand from there
-        if os.environ.get("SA_DKDV3_RING_ACC"):
-            return self.ar((224 if r < 8 else 192 - 32) + 4 * r + lo, n)
         if r < 8:
             return self.vr(112 + 4 * r + lo, n)
         return self.ar(192 + 4 * (r - 8) + lo, n)

@@ -36,8 +36,6 @@ Register map (D = 128):
 Run:  python3 gen_dq3_asm.py > sa_dq3_asm.inc   (the Makefile does this)
 """
 
-import os
-RING_ACC = bool(os.environ.get("SA_DQ3_RING_ACC"))   # experiment: fragment ring in a[128:159], Q fragments of block 0 in v[160:191]
 RING = 8
 PF = RING - 1          # fragments between a read and its use
 NFRAG = 24             # fragments per iteration: 8 K rows, 8 V rows (alternating), 8 K transposed
@@ -60,8 +58,6 @@ def DQ(qb, m):
 
 
 def QF(qb, g):
-    if RING_ACC and qb == 0:
-        return vr(160 + 4 * g, 4)
     return ar(128 + 32 * qb + 4 * g, 4)
 
 
@@ -83,8 +79,6 @@ def DSB(buf, qb, half, w=None):
 
 
 def RG(r, lo=0, n=4):
-    if RING_ACC:
-        return ar(128 + 4 * r + lo, n)
     return vr(160 + 4 * r + lo, n)
 
 
@@ -284,8 +278,6 @@ def generate(dt):
     g = Gen(dt)
     # ---- prologue: scalars, scores and delta - dP of block 0, ring entries of the first iteration -------
     pro = [f"v_readfirstlane_b32 s{40 + i}, v{160 + i}" for i in range(len(SCALARS))]
-    if RING_ACC:
-        pro += [f"v_accvgpr_read_b32 v{160 + i}, a{128 + i}" for i in range(32)] + ["s_nop 1"]
     g.out = pro
     for half in range(2):          # row fragments 4*half .. 4*half+3 of K and V: 8 ring entries at a time
         for x in range(8):
