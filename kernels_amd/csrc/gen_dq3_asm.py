@@ -32,6 +32,7 @@ Register map (D = 128):
   asynchronous loads  s49 -inf  s50, s51: a block inside [s50, s51) lies inside the window of every query of
   this wave  s[52:55], s[56:59] buffer resources of K and V  s60, s61 their running byte offsets  s62, s63 bytes
   between a wave's load instructions  s64, s65 bytes between tiles  s66..s69 temporaries
+  s70, s71 first key tile of this wave's own window and one past its last (s41: of the workgroup's window)
 
 Run:  python3 gen_dq3_asm.py > sa_dq3_asm.inc   (the Makefile does this)
 """
@@ -253,7 +254,7 @@ class Gen:
 
 SCALARS = ["sl2e", "kt1", "t", "kb", "st0", "st1", "st2", "st3", "wave_tile", "ninf", "lo_max", "hi_min",
            "rk0", "rk1", "rk2", "rk3", "rv0", "rv1", "rv2", "rv3", "soff_k", "soff_v", "istep_k", "istep_v",
-           "tstep_k", "tstep_v"]          # v160 + i  ->  s40 + i
+           "tstep_k", "tstep_v", "wfirst", "wend"]          # v160 + i  ->  s40 + i
 
 
 def issue_tile():
@@ -276,8 +277,31 @@ def issue_tile():
 def generate(dt):
     L = lambda name: f"{name}_{dt}_%="
     g = Gen(dt)
+    # tile hand-over of an even iteration: tile s42 + 1 must have landed in every wave's share before its
+    # rows are read (slot 34 on); the stage of tile s42 - 2 (s47), which nobody reads any more, takes tile s42 + 2
+    def mid(lab):
+        return ["s_add_i32 s66, s42, 1",
+                "s_cmp_ge_i32 s66, s41",
+                f"s_cbranch_scc1 Lskip_{lab}",
+                "s_waitcnt vmcnt(0)",
+                "s_barrier",
+                "s_add_i32 s66, s42, 2",
+                "s_cmp_ge_i32 s66, s41",
+                f"s_cbranch_scc1 Lskip_{lab}"] + issue_tile() + [f"Lskip_{lab}:"]
     # ---- prologue: scalars, scores and delta - dP of block 0, ring entries of the first iteration -------
-    pro = [f"v_readfirstlane_b32 s{40 + i}, v{160 + i}" for i in range(len(SCALARS))]
+    sreg = lambda i: 40 + i if i < 26 else 70 + (i - 26)     # s66..s69 are temporaries
+    pro = [f"v_readfirstlane_b32 s{sreg(i)}, v{160 + i}" for i in range(len(SCALARS))]
+    rotate = ["s_mov_b32 s66, s44", "s_mov_b32 s44, s45", "s_mov_b32 s45, s46", "s_mov_b32 s46, s47", "s_mov_b32 s47, s66"]
+    # Tiles of the workgroup's window that lie before this wave's own window (s70 = its first tile): no arithmetic,
+    # only the wave's part in the hand-over of every tile (its share of the loads, the barrier).  The same after
+    # the wave's last tile (s71 = one past it).
+    pro += [L("Lin") + ":",
+            "s_cmp_ge_i32 s42, s70",
+            "s_cbranch_scc1 " + L("Lin_done")] + mid(L("i")) + [
+            "s_add_i32 s42, s42, 1"] + rotate + [
+            "s_branch " + L("Lin"),
+            L("Lin_done") + ":",
+            "s_lshl_b32 s43, s42, 6"]
     g.out = pro
     for half in range(2):          # row fragments 4*half .. 4*half+3 of K and V: 8 ring entries at a time
         for x in range(8):
@@ -298,17 +322,6 @@ def generate(dt):
     for f in range(PF):
         g.fetch(NFRAG + f, f, 0)
     text = g.out
-    # tile hand-over of an even iteration: tile s42 + 1 must have landed in every wave's share before its
-    # rows are read (slot 34 on); the stage of tile s42 - 2 (s47), which nobody reads any more, takes tile s42 + 2
-    def mid(lab):
-        return ["s_add_i32 s66, s42, 1",
-                "s_cmp_ge_i32 s66, s41",
-                f"s_cbranch_scc1 Lskip_{lab}",
-                "s_waitcnt vmcnt(0)",
-                "s_barrier",
-                "s_add_i32 s66, s42, 2",
-                "s_cmp_ge_i32 s66, s41",
-                f"s_cbranch_scc1 Lskip_{lab}"] + issue_tile() + [f"Lskip_{lab}:"]
     k = 1
     first = g.body(k, 0, L("f"), with_dq=False, mid=mid(L("f")))
     k += 1
@@ -325,8 +338,8 @@ def generate(dt):
     text += b1
     text += ["s_add_i32 s42, s42, 1",
              "s_add_i32 s43, s43, 32",
-             "s_mov_b32 s66, s44", "s_mov_b32 s44, s45", "s_mov_b32 s45, s46", "s_mov_b32 s46, s47", "s_mov_b32 s47, s66",
-             "s_cmp_ge_i32 s42, s41",
+             *rotate,
+             "s_cmp_ge_i32 s42, s71",
              "s_cbranch_scc1 " + L("Lend")]
     text += b0
     text += ["s_branch " + L("Lloop"),
@@ -344,8 +357,13 @@ def generate(dt):
         text.append(f"s_waitcnt lgkmcnt({min(n, 15)})")
         for qb in range(2):
             text.append(f"{g.mfma} {DQ(qb, m)}, {RG(x)}, {DSB(1, qb, half)}, {DQ(qb, m)}")
-    text += ["s_nop 15", "s_nop 15", "s_nop 15", "s_nop 15",
-             "s_branch " + L("Lout")]
+    text += ["s_nop 15", "s_nop 15", "s_nop 15", "s_nop 15"]
+    # tiles of the workgroup's window after this wave's last one
+    text += [L("Lfin") + ":",
+             "s_cmp_ge_i32 s42, s41",
+             "s_cbranch_scc1 " + L("Lout")] + mid(L("x")) + [
+             "s_add_i32 s42, s42, 1"] + rotate + [
+             "s_branch " + L("Lfin")]
     text += g.tails
     text.append(L("Lout") + ":")
     name = f"SA_DQ3_128_{dt.upper()}"
