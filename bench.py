@@ -427,6 +427,33 @@ def measure_workload(name, dev, steps, warmup, kernel_iters, zeros=False, compil
     median_ms = per_step[len(per_step) // 2] if len(per_step) % 2 else \
         0.5 * (per_step[len(per_step) // 2 - 1] + per_step[len(per_step) // 2])
 
+    # the same step captured once into a HIP graph and replayed: what a caller pays who takes the Python and
+    # dispatcher work out of the loop (the library records nothing but its kernels into the graph)
+    graph_ms = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        q.grad = k.grad = v.grad = None
+        with torch.cuda.graph(graph):
+            out = streaming_attention(q, k, v, w["lens"], C, R)
+            out.backward(w["d_o"])
+        for _ in range(warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t2) * 1e3 / steps
+        del graph
+    except Exception as e:      # reported, never fatal for the headline figures
+        print(f"graph replay of {name} not measured: {e!r}", file=sys.stderr)
+
     compiled_ms = None
     if compiled:
         # the same step through the torch.compile'd wrapper that the reference puts around the op
@@ -480,7 +507,7 @@ def measure_workload(name, dev, steps, warmup, kernel_iters, zeros=False, compil
     q.grad = k.grad = v.grad = None
     return {"inputs": w, "pairs": P, "flops_step": flops_step, "step_bytes": step_bytes, "ms_per_step": ms_per_step,
             "value": value, "median_ms": median_ms, "median_steps": n_med, "compiled_wrapper_ms_per_step": compiled_ms,
-            "kernel_ms": kt, "kernel_variants": variants,
+            "graph_replay_ms_per_step": graph_ms, "kernel_ms": kt, "kernel_variants": variants,
             "kernel_tflops": {n: kernel_flops[n] / (kt[n] * 1e-3) / 1e12 for n in kernel_flops},
             "kernel_gbs": {n: kernel_bytes[n] / (kt[n] * 1e-3) / 1e9 for n in kernel_bytes}, "roofline": roofline}
 
@@ -545,6 +572,7 @@ def main():
         "value": m["value"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": m["ms_per_step"], "median_ms": m["median_ms"], "median_steps": m["median_steps"],
         "compiled_wrapper_ms_per_step": m["compiled_wrapper_ms_per_step"],
+        "graph_replay_ms_per_step": m["graph_replay_ms_per_step"],
         "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None,
         "dtype": {"bfloat16": "bf16", "float16": "f16", "float32": "f32"}[w["dtype"]],
@@ -577,6 +605,7 @@ def main():
             dom = o["roofline"]["kernel"]
             others[name] = {
                 "ms_per_step": o["ms_per_step"], "median_ms": o["median_ms"], "steps": steps,
+                "graph_replay_ms_per_step": o["graph_replay_ms_per_step"],
                 "effective_tflops": o["value"], "pct_of_bf16_mfma_peak": 100.0 * o["value"] / PEAK_BF16_TFLOPS,
                 "step_hbm_gbs": o["step_bytes"] / (o["ms_per_step"] * 1e-3) / 1e9,
                 "kernel_ms": o["kernel_ms"], "kernel_variants": o["kernel_variants"], "dominant_kernel": dom,

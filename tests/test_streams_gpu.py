@@ -90,3 +90,54 @@ def test_forward_on_two_overlapping_streams(pipelined_forward):
         assert torch.equal(o, want1[0]) and torch.equal(lse, want1[1])
     for o, lse in got2:
         assert torch.equal(o, want2[0]) and torch.equal(lse, want2[1])
+
+
+@pytest.mark.parametrize("dtype,D_,C,R", [(torch.bfloat16, 128, 256, 8), (torch.float16, 128, 64, 1), (torch.bfloat16, 64, 128, 4),
+                                         (torch.float32, 32, 16, 3)], ids=str)
+def test_step_replayed_from_a_graph_equals_the_eager_step(dtype, D_, C, R):
+    """Forward and backward through the public function, captured once and replayed three times with eager steps in
+    between: every replay must reproduce the eager gradients bit for bit (a graph must hold nothing but the
+    library's kernels and torch's own fill and copy kernels)."""
+    from streaming_attention import streaming_attention
+
+    dev = torch.device("cuda:0")
+    B, H, T = 3, 4, 1500
+    g = torch.Generator(device=dev).manual_seed(21)
+    q, k, v, d_o = ((torch.randn(B, H, T, D_, generator=g, device=dev) * 0.5).to(dtype) for _ in range(4))
+    lens = torch.tensor([1500, 700, 64], dtype=torch.int32, device=dev)
+    for t in (q, k, v):
+        t.requires_grad_()
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        out = streaming_attention(q, k, v, lens, C, R)
+        out.backward(d_o)
+        return out
+
+    want_o = step().detach().clone()
+    want = [t.grad.clone() for t in (q, k, v)]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    q.grad = k.grad = v.grad = None
+    with torch.cuda.graph(graph):
+        out_g = streaming_attention(q, k, v, lens, C, R)
+        out_g.backward(d_o)
+    grads_g = [q.grad, k.grad, v.grad]          # static tensors of the graph
+    for _ in range(3):
+        for t in grads_g:
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want_o)
+        for got, w_ in zip(grads_g, want):
+            assert torch.equal(got, w_)
+        # eager work of the same kind between the replays, on fresh gradient tensors
+        keep = [q.grad, k.grad, v.grad]
+        step()
+        q.grad, k.grad, v.grad = keep
+        torch.cuda.synchronize()
