@@ -28,7 +28,7 @@
  *     mutex) and the variants pinned through sa_tune_override() (atomics; a measurement and test
  *     hook that no product caller needs).  Because of the former, the first call of each kernel
  *     shape on a device must be made outside a HIP graph capture.
- *   - The 16-bit dK/dV kernels at D >= 64 multiply K by -sm_scale*log2(e) and round the product to the
+ *   - The 16-bit dK/dV kernels at D >= 32 multiply K by -sm_scale*log2(e) and round the product to the
  *     element type before the score MFMA (what the reference does for prescale_qk=True,
  *     src/streaming_attention/kernel.py:1065-1066), whatever `prescale_qk` the caller of the Python
  *     operator passed: their probabilities differ from the forward's by about |score| * 2^-9 (bf16) /
@@ -102,7 +102,7 @@ int sa_bwd_dkdv(const void* q, const void* k, const void* v,
 
 /* Whole backward on one stream; `delta` is a caller-provided [B,H,T] float32 workspace that holds
  * rowsum(O * dO) afterwards.  For float32 and for head dimensions 16 and 32 this is sa_bwd_delta +
- * sa_bwd_dkdv + sa_bwd_dq.  For float16 / bfloat16 at head dimensions 64, 128 and 256 the dQ kernel
+ * sa_bwd_dkdv + sa_bwd_dq.  For float16 / bfloat16 at head dimensions 32, 64, 128 and 256 the dQ kernel
  * forms the row sums itself from the dO rows it holds anyway (it reads O once more and writes
  * `delta` for the dK/dV kernel, which runs after it), so the separate pass over O and dO -- the
  * reference's `_streaming_attn_bwd_precompute` launch, kernel.py:433-514 -- is not launched; the

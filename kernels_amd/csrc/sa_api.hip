@@ -22,7 +22,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // strides are element counts; dim stride 1, the others whole 16-byte vectors.  The 16-bit kernels
-// for D >= 64 address the rows of one (batch, head) slice with 32-bit byte offsets through a
+// for D >= 32 address the rows of one (batch, head) slice with 32-bit byte offsets through a
 // buffer descriptor; the others compute 64-bit addresses and have no such limit.  A zero stride along
 // T (one row repeated) is refused: no caller needs it and no test covers it.
 int check_layout(const void* p, const int64_t* s, int dtype, int T, int D) {
@@ -33,7 +33,7 @@ int check_layout(const void* p, const int64_t* s, int dtype, int T, int D) {
   for (int i = 0; i < 3; ++i)
     if (s[i] % vec != 0) return SA_ERR_LAYOUT;
   if (s[2] < 0 || (s[2] == 0 && T > 1)) return SA_ERR_LAYOUT;
-  const bool offsets32 = dtype != SA_DTYPE_F32 && D >= 64;
+  const bool offsets32 = dtype != SA_DTYPE_F32 && D >= 32;
   if (offsets32 && ((int64_t)T + 1024) * s[2] * 2 >= (int64_t(1) << 32)) return SA_ERR_TOO_LARGE;
   return SA_OK;
 }

@@ -63,7 +63,7 @@ template <> struct Elem<float> {
 };
 
 // LDS tile geometry.  Two layouts:
-//  * swizzled (16-bit types, D >= 64): rows are stored unpadded and the 16-byte chunk index
+//  * swizzled (16-bit types, D >= 32): rows are stored unpadded and the 16-byte chunk index
 //    inside a row is XOR-ed with a permutation of the low row bits, chosen so that both access
 //    patterns of the kernels spread over all 64 banks: 16 lanes reading the same chunk of 16
 //    consecutive rows (row-major fragments), and 32 lanes reading a 4-row x 64-byte patch
@@ -79,7 +79,7 @@ template <> struct Elem<float> {
 template <typename T, int D> struct TileGeom {
   static constexpr int VEC = Elem<T>::VEC;
   static constexpr int DP = D < 32 ? 32 : D;
-  static constexpr bool SWZ = SA_SWIZZLE && Elem<T>::HALF && D >= 64;
+  static constexpr bool SWZ = SA_SWIZZLE && Elem<T>::HALF && D >= 32;
   static constexpr int PITCH = SWZ ? D : DP + SA_PAD_VECS * VEC;
   static constexpr int NF = D / (2 * VEC);   // row fragments per lane
   static constexpr int DB = DP / 32;         // 32-wide blocks along D
@@ -89,7 +89,8 @@ template <typename T, int D> struct TileGeom {
   SA_DEV static int swz(int row) {
     if constexpr (!SWZ) return 0;
     else if constexpr (CPR >= 16) return ((row & 3) << 2) | ((row >> 2) & 3);
-    else return ((row >> 2) & 1) | (((row >> 3) & 1) << 1) | (((row >> 1) & 1) << 2);   // CPR == 8
+    else if constexpr (CPR == 8) return ((row >> 2) & 1) | (((row >> 3) & 1) << 1) | (((row >> 1) & 1) << 2);
+    else return (row >> 2) & 3;   // CPR == 4: four rows fill the 64 banks, rows 4 apart must differ
   }
   // element offset of (row, element col) inside a tile
   SA_DEV static int off(int row, int col) {

@@ -260,7 +260,7 @@ template <int D> static int dkdv3_launch(BwdParams p, hipStream_t st) {
 // wave pairs: 8 waves (two per SIMD) own 128 keys
 template <int D> static int dkdv_split_launch(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
-  if constexpr (C::fwd2(D) && D <= 128) {
+  if constexpr (C::fwd2(D) && D >= 64 && D <= 128) {
     constexpr int TKB = 128, TQ = 64, NST = 3, NW = 8;
     // tile stages followed by the pairs' exchange slots; the epilogue's row patches reuse the stages
     constexpr size_t stages = (size_t)NST * (2 * TQ * D * sizeof(ElemT) + 2 * TQ * sizeof(float));
@@ -282,7 +282,9 @@ template <int D> static int dkdv_split_launch(BwdParams p, hipStream_t st) {
 template <int D> static int dkdv_d(BwdParams p, hipStream_t st) {
   using C = Cfg<ElemT>;
   if constexpr (C::fwd2(D)) {
-    if (launch_choice(D, p.C, p.R).dkdv == DKDV_SPLIT) return dkdv_split_launch<D>(p, st);
+    if constexpr (D >= 64) {   // a 64-byte row splits over four waves' copies, not over eight
+      if (launch_choice(D, p.C, p.R).dkdv == DKDV_SPLIT) return dkdv_split_launch<D>(p, st);
+    }
     // The pipelined kernel (head dimension 128) makes every wave walk the whole window of its
     // workgroup's 128 keys; that wastes nothing once a chunk holds at least those 128 keys.  Smaller
     // chunks go to the kernel whose waves skip the query tiles outside their own 32 keys' windows.

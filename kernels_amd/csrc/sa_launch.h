@@ -111,7 +111,7 @@ template <typename T> struct Cfg {
 #ifdef SA_FWD2_DISABLE
   static constexpr bool fwd2(int) { return false; }
 #else
-  static constexpr bool fwd2(int D) { return sizeof(T) == 2 && (D == 64 || D == 128 || D == 256); }
+  static constexpr bool fwd2(int D) { return sizeof(T) == 2 && (D == 32 || D == 64 || D == 128 || D == 256); }
 #endif
 #ifdef SA_FWD_TK16
   static constexpr int FWD_TK = sizeof(T) == 4 ? 32 : SA_FWD_TK16;

@@ -8,7 +8,7 @@ compatibility and do not change the result: kernel variants are read from a tabl
 on MI355X (head dimension, context_size class, window class), all accumulation is fp32, and
 where the scale is applied is fixed per kernel: in float32 inside the exp2 argument in the forward
 and dQ kernels (at least as accurate as either setting of ``prescale_qk``), folded into K and
-rounded to the element type in the 16-bit dK/dV kernels at head dimensions 64 and up (what the
+rounded to the element type in the 16-bit dK/dV kernels at head dimensions 32 and up (what the
 reference does under ``prescale_qk=True``, kernel.py:1065-1066).
 """
 from __future__ import annotations
@@ -36,11 +36,11 @@ def _dtype_id(dtype: torch.dtype) -> int:
 def _kernel_layout(t: torch.Tensor) -> torch.Tensor:
     """Return ``t`` itself when the kernels can read it in place (unit stride along the head
     dimension, every other stride and the base address a multiple of 16 bytes, a non-zero stride
-    along T), otherwise a contiguous copy.  The 16-bit kernels for head dimensions 64 and up
+    along T), otherwise a contiguous copy.  The 16-bit kernels for head dimensions 32 and up
     address the rows of one (batch, head) slice with 32-bit byte offsets (a contiguous tensor is
     within that range up to tens of millions of positions); the other kernels have no such limit."""
     es = t.element_size()
-    offsets32 = es == 2 and t.shape[-1] >= 64
+    offsets32 = es == 2 and t.shape[-1] >= 32
     if t.is_contiguous() and t.data_ptr() % _VEC_BYTES == 0 and t.shape[-1] * es % _VEC_BYTES == 0 \
             and (not offsets32 or (t.shape[-2] + 1024) * t.shape[-1] * es < 2**32):
         return t          # the common case, without looking at every stride

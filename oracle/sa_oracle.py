@@ -86,7 +86,7 @@ def dense_f64(q, k, v, lens, context_size, back_contexts, sm_scale=None, d_out=N
     softmax denominator sums the rounded probabilities, and O is rounded before delta is formed.
     The difference between the two evaluations is the error that rounding alone causes.
     ``prescaled_k`` (with ``round_dtype``) also models the scores of the 16-bit dK/dV kernels for head
-    dimensions 64 and up, which fold -scale*log2(e) into K and round the product to the element type
+    dimensions 32 and up, which fold -scale*log2(e) into K and round the product to the element type
     before the score product (the reference's prescale_qk=True, kernel.py:1065-1066): dK and dV are then
     formed from probabilities exp2(q . round(k*scale*log2e) - lse), dQ from the unrounded scale."""
     qn, kn, vn = (t.detach().cpu().double() for t in (q, k, v))

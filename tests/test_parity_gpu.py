@@ -355,7 +355,7 @@ def check_rounding_aware(q, k, v, d_o, lens, C, R, dtype, sm_scale=None, record=
     o, lse, dq, dk, dv = run_kernel(q, k, v, d_o, lens, C, R, **kw)
     exact = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=sm_scale, d_out=d_o)
     rounded = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=sm_scale, d_out=d_o, round_dtype=dtype,
-                                  prescaled_k=q.shape[-1] >= 64)
+                                  prescaled_k=q.shape[-1] >= 32)
     for name, got in (("O", o), ("dQ", dq), ("dK", dk), ("dV", dv)):
         assert_close_rounding_aware(name, got, exact[name], rounded[name], dtype)
         mx, rel, fro = error_report(got, exact[name])
@@ -463,7 +463,7 @@ def test_random_problems(seed):
         # the bar allows for the rounding of P and dS, and of the pre-scaled K in the dK/dV kernels,
         # as a float64 evaluation with those roundings shows it (see check_rounding_aware)
         rnd = sa_oracle.dense_f64(q, k, v, lens, C, R, sm_scale=scale, d_out=d_o, round_dtype=dtype,
-                                  prescaled_k=D >= 64)
+                                  prescaled_k=D >= 32)
         for name, got in results:
             assert_close_rounding_aware(name, got, ref[name], rnd[name], dtype)
     if dtype != torch.float32:
